@@ -5,7 +5,12 @@ Two kinds of per-sequence memory share one sequence table:
 * **pages**: per caching attention layer either one tensor [blocks, BLK,
   width] (latent attention: the normalised latent row and the rotated shared
   key part of each token) or a key tensor [blocks, BLK, heads x size] and a
-  transposed value tensor [blocks, heads x size, BLK] (``kv``). The pages of all layers follow ONE block table per sequence,
+  transposed value tensor [blocks, heads x size, BLK] (``kv``), or key and
+  value tensors that are both [blocks, BLK, heads x size] (``kv_rows``). The
+  keys of these dictionaries are whatever the model's step function uses to
+  find its storage: a layer index, or the index of a layer RUN when a model
+  runs a stretch of layers several times and each pass caches for itself. The
+  pages of all of them follow ONE block table per sequence,
   handed out by the same block pool the Llama KV cache uses (native
   ``BlockPool``);
 * **state slots**: one slot per live sequence (the last slot is the write
@@ -103,6 +108,11 @@ class HybridCache:
         self.kv = {li: (torch.zeros(num_blocks, block_size, kw, dtype=dtype, device=dev),
                         torch.zeros(num_blocks, vw, block_size, dtype=dtype, device=dev))
                    for li, (kw, vw) in spec.get("kv", {}).items()}
+        # key pages and value pages in the same row-major layout (softmax
+        # attention: its kernels stage both through LDS tile by tile)
+        self.kv_rows = {li: (torch.zeros(num_blocks, block_size, kw, dtype=dtype, device=dev),
+                             torch.zeros(num_blocks, block_size, vw, dtype=dtype, device=dev))
+                        for li, (kw, vw) in spec.get("kv_rows", {}).items()}
         # named per-sequence rows
         self.rows = {li: {name: torch.zeros(max_seqs + 1, *shape, dtype=torch.float32, device=dev)
                           for name, shape in named.items()}
@@ -123,6 +133,6 @@ class HybridCache:
 
     def nbytes(self) -> int:
         ts = [*self.latent.values(), *self.state.values()]
-        ts += [t for pair in self.kv.values() for t in pair]
+        ts += [t for pair in (*self.kv.values(), *self.kv_rows.values()) for t in pair]
         ts += [t for named in self.rows.values() for t in named.values()]
         return sum(t.numel() * t.element_size() for t in ts)

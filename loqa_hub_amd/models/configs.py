@@ -259,10 +259,14 @@ class FeedForwardConfig:
     shared_ff: int = 0              # 0: no shared expert
     # "swiglu": down(silu(gate x) * (up x)); "relu2": down(relu(up x)^2), no gate
     act: str = "swiglu"
+    # "swiglu" / "geglu" (the tanh form of GELU on the gate) for dense layers
     # router: "softmax_all" scores every output and weighs by the plain score;
     # "softmax_top" takes the largest logits (+ bias) and weighs by the softmax
-    # over the chosen ones only
+    # over the chosen ones only; "sigmoid" scores every output by the logistic
+    # function of its logit and weighs by the plain score
     router: str = "softmax_all"
+    # a group of experts ranks by the sum of its ``group_rank`` best scores
+    group_rank: int = 1
 
 
 @dataclass(frozen=True)
@@ -400,3 +404,145 @@ def sodonex_config_from_json(d: dict, name: str = "sodonex") -> SodonexConfig:
         layers.append(HybridLayerConfig(kind, mixer, mlp))
     return SodonexConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
                          float(d["residual_mult"]), float(d["embedding"]["scale"]), tuple(layers))
+
+
+# --------------------------------------------------------------------------
+# Movinex: a pre-norm decoder (RMS norms with weights stored around zero, a
+# learned per-coordinate scale on every sublayer output) whose config.json
+# lists its layers; a stretch of layers may run several times in a row with the
+# same weights. Mixers: softmax attention (full causal with a position-dependent
+# query temperature, or sliding-window with kept first tokens, interleaved
+# rotary, score soft-capping, keys doubling as values and an output gate) and
+# Mamba-2 state-space layers. Feed-forwards: dense GeGLU or a sigmoid-routed
+# mixture of SwiGLU experts. Every size and constant comes from config.json or
+# a tensor's shape.
+@dataclass(frozen=True)
+class SoftmaxAttnConfig:
+    heads: int
+    kv_heads: int
+    dim: int                        # query / key size per head
+    vdim: int                       # value size per head
+    scale: float
+    bias: bool = False              # q / k / v projections carry biases
+    values_from_keys: bool = False  # no value projection: v = k as projected
+    gate: bool = False              # heads' outputs times sigmoid(W_g h), per entry
+    rot: RotaryConfig | None = None     # interleaved pairs on the first rot.dims entries
+    q_temp: tuple | None = None     # (coef, every): q *= 1 + coef ln(floor((p + 1) / every) + 1)
+    softcap: float = 0.0            # score <- cap tanh(score / cap); 0: none
+    window: int = 0                 # key j visible if p - j < window ...; 0: every earlier key
+    keep_first: int = 0             # ... or j < keep_first
+
+
+@dataclass(frozen=True)
+class Mamba2Config:
+    heads: int
+    vdim: int                       # channels per head
+    state: int                      # N
+    groups: int                     # B / C groups shared by neighbouring heads
+    taps: int                       # causal convolution on x | B | C
+    norm_groups: int                # the gated output is RMS-normed in this many parts
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
+class LoopConfig:
+    start: int
+    stop: int                       # layers start .. stop - 1 ...
+    times: int                      # ... run this many times in a row
+
+
+@dataclass(frozen=True)
+class MovinexConfig:
+    name: str
+    vocab_size: int
+    d_model: int
+    norm_eps: float
+    logit_scale: float
+    layers: tuple
+    loop: LoopConfig | None = None
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list[tuple[int, bool]]:
+        """The layers in execution order as (layer index, first of a pass of the
+        repeated stretch); every run has a cache or state of its own."""
+        n = len(self.layers)
+        if self.loop is None:
+            return [(i, False) for i in range(n)]
+        lp = self.loop
+        out = [(i, False) for i in range(lp.start)]
+        for _ in range(lp.times):
+            out += [(i, i == lp.start) for i in range(lp.start, lp.stop)]
+        return out + [(i, False) for i in range(lp.stop, n)]
+
+
+def movinex_config_from_json(d: dict, name: str = "movinex") -> MovinexConfig:
+    layers = []
+    for i, L in enumerate(d["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind in ("attention", "attention_2"):
+            second = kind == "attention_2"
+            r, qt, mk = m.get("rot"), m.get("q_temp"), m.get("mask") or {}
+            mixer = SoftmaxAttnConfig(
+                int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                float(m["scale"]), bias=not second, values_from_keys=second, gate=second,
+                rot=RotaryConfig(int(r["dims"]), float(r["base"])) if r else None,
+                q_temp=(float(qt["coef"]), int(qt["every"])) if qt else None,
+                softcap=float(m.get("softcap") or 0.0), window=int(mk.get("size") or 0),
+                keep_first=int(mk.get("keep_first") or 0))
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError(f"layer {i}: {mixer.heads} heads do not split over "
+                                 f"{mixer.kv_heads} key/value heads")
+            if mixer.values_from_keys and mixer.vdim != mixer.dim:
+                raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim")
+            if mixer.rot and (mixer.rot.dims % 2 or not 0 <= mixer.rot.dims <= mixer.dim):
+                raise ValueError(f"layer {i}: rot.dims {mixer.rot.dims} does not fit a head")
+            if mixer.q_temp and mixer.q_temp[1] < 1:
+                raise ValueError(f"layer {i}: q_temp.every must be positive")
+        elif kind == "mamba2":
+            mixer = Mamba2Config(int(m["heads"]), int(m["vdim"]), int(m["state"]),
+                                 int(m.get("groups", 1)), int(m["conv"]),
+                                 int(m.get("norm_groups", 1)))
+            if mixer.heads % mixer.groups or mixer.inner % mixer.norm_groups or mixer.taps < 1:
+                raise ValueError(f"layer {i}: heads, groups and norm_groups do not fit")
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = L.get("mlp")
+        if not f:
+            mlp = None
+        elif f["kind"] == "dense":
+            mlp = FeedForwardConfig("dense", int(f["ff"]), act="geglu")
+        elif f["kind"] == "moe":
+            r = f["router"]
+            g = r.get("groups") or {}
+            mlp = FeedForwardConfig("moe", int(f["expert"]["ff"]), int(r["experts"]), 0,
+                                    int(r["top"]), int(g.get("count", 1)),
+                                    int(g.get("keep", g.get("count", 1))), router="sigmoid",
+                                    group_rank=2)
+            if mlp.experts % mlp.groups or not 0 < mlp.keep <= mlp.groups:
+                raise ValueError(f"layer {i}: {mlp.experts} experts do not split into "
+                                 f"{mlp.groups} groups")
+            if not 0 < mlp.top <= mlp.keep * (mlp.experts // mlp.groups):
+                raise ValueError(f"layer {i}: top {mlp.top} exceeds the eligible experts")
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(HybridLayerConfig(kind, mixer, mlp))
+    lp = d.get("loop")
+    loop = None
+    if lp:
+        loop = LoopConfig(int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+        if not 0 <= loop.start <= loop.stop <= len(layers) or loop.times < 1:
+            raise ValueError("loop: start, stop and times do not fit the layer list")
+        if loop.start == loop.stop:
+            loop = None
+    return MovinexConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
+                         float(d.get("logit_scale", 1.0)), tuple(layers), loop)

@@ -217,10 +217,11 @@ _SEQMIX_SIGS = {
     "loqa_rope_pairs": [_vp, _l, _l, _i, _i, _i, _i, _vp, _vp, _i, _vp],
     "loqa_latent_prefill": [_vp, _l, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _vp],
     "loqa_lightning_prep": [_vp, _i, _l, _i, _i, _vp, _vp],
-    "loqa_lightning_scan": [_vp, _l, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
-    "loqa_gated_rmsnorm": [_vp, _vp, _vp, _i, _l, _f, _vp, _i, _i, _i, _vp],
-    "loqa_silu_mul_any": [_vp, _i, _i, _i, _vp, _vp],
-    "loqa_moe_route": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp],
+    "loqa_state_scan": [_vp, _l, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp,
+                        _vp, _i, _i, _vp],
+    "loqa_gated_rmsnorm": [_vp, _vp, _vp, _i, _l, _f, _vp, _i, _i, _i, _i, _i, _vp],
+    "loqa_act_mul_any": [_vp, _i, _i, _i, _i, _vp, _vp],
+    "loqa_moe_route": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp],
     "loqa_moe_plan": [_vp, _i, _i, _vp, _vp],
     "loqa_moe_grouped_gemm": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp],
     "loqa_moe_combine": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
@@ -233,6 +234,14 @@ _SEQMIX_SIGS = {
                                _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp],
     "loqa_scalar_rms_add": [_vp, _vp, _i, _f, _f, _vp, _i, _i, _vp],
     "loqa_scalar_rms_norm": [_vp, _vp, _f, _f, _vp, _i, _i, _vp],
+    "loqa_rms1p_norm": [_vp, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+    "loqa_scaled_add_rms1p": [_vp, _vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+    "loqa_qk_prep_append": [_vp, _i, _l, _i, _i, _i, _i, _i, _vp, _i, _i, _f, _f, _i, _vp, _vp,
+                            _vp, _i, _i, _vp, _vp, _i, _vp],
+    "loqa_window_attention": [_vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _l, _f, _f,
+                              _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp],
+    "loqa_mamba2_prep": [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp,
+                         _vp, _i, _i, _vp, _vp, _vp],
 }
 _seqmix = None
 

@@ -31,6 +31,19 @@ def layernorm(x, w, b, eps, residual=None):
     return y.to(x.dtype)
 
 
+def gelu_tanh(z):
+    """0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
+    return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+
+
+def act_mul(x, act: str = "silu"):
+    """[gate | up] -> act(gate) * up in f32, rounded to x's dtype."""
+    F = x.shape[-1] // 2
+    g, u = x[..., :F].float(), x[..., F:].float()
+    a = gelu_tanh(g) if act == "gelu_tanh" else torch.nn.functional.silu(g)
+    return (a * u).to(x.dtype)
+
+
 def silu_mul(x):
     F = x.shape[-1] // 2
     g, u = x[..., :F].float(), x[..., F:].float()
@@ -696,18 +709,28 @@ def latent_attention(qa, qr, cache, cu_q, ctx_lens, block_tables, positions, cos
     return out
 
 
-def lightning_scan(qkv, H: int, D: int, Dv: int, state, state_slots, cu_q, positions, decay):
-    """Decayed linear attention, token by token: S <- decay_h S + k v^T,
-    o = S^T q with q, k, v = silu of the [q | k | v] columns of ``qkv``. The
-    state [slots, H, D, Dv] (f32) is read at the sequence's slot (zero when
-    the step's first position is 0) and written back. Returns o f32 [T, H Dv]."""
-    T = qkv.shape[0]
-    a = torch.nn.functional.silu(qkv[:, :2 * H * D + H * Dv].float())
-    q, k = a[:, :H * D].view(T, H, D), a[:, H * D:2 * H * D].view(T, H, D)
-    v = a[:, 2 * H * D:].view(T, H, Dv)
-    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=qkv.device)
+def state_scan(act, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int, hpg: int, state,
+               state_slots, cu_q, positions, decay=None, tok=None, skip=None):
+    """Linear recurrence with a carried matrix state, token by token in f32:
+
+        S <- a S + k (c v)^T,    o = S^T q + skip_h v
+
+    per sequence and head, with a = ``decay[h]`` (constant) or ``tok[t, h, 0]``
+    (per token) and c = 1 or ``tok[t, h, 1]``. ``act`` f32 [T, W] holds the
+    inputs: head h reads q at ``q_off + (h // hpg) D``, k at ``k_off + (h //
+    hpg) D`` (``hpg`` neighbouring heads share one q / k group) and v at
+    ``v_off + h Dv``. The state [slots, H, D, Dv] is read at the sequence's
+    slot (zero when the step's first position is 0) and written back.
+    Returns o f32 [T, H Dv]."""
+    T = act.shape[0]
+    a = act.float()
+    hg = torch.arange(H, device=act.device) // hpg
+    cols = torch.arange(D, device=act.device)
+    q = a[:, (q_off + hg[:, None] * D + cols[None, :]).reshape(-1)].view(T, H, D)
+    k = a[:, (k_off + hg[:, None] * D + cols[None, :]).reshape(-1)].view(T, H, D)
+    v = a[:, v_off:v_off + H * Dv].view(T, H, Dv)
+    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=act.device)
     cu = cu_q.tolist()
-    lam = decay.float()[:, None, None]
     for b in range(len(cu) - 1):
         q0, q1 = cu[b], cu[b + 1]
         if q1 == q0:
@@ -715,37 +738,61 @@ def lightning_scan(qkv, H: int, D: int, Dv: int, state, state_slots, cu_q, posit
         slot = int(state_slots[b])
         S = torch.zeros_like(state[slot]) if int(positions[q0]) == 0 else state[slot].clone()
         for t in range(q0, q1):
-            S = lam * S + k[t][:, :, None] * v[t][:, None, :]
+            lam = decay.float()[:, None, None] if tok is None else tok[t, :, 0].float()[:, None, None]
+            vt = v[t] if tok is None else v[t] * tok[t, :, 1].float()[:, None]
+            S = lam * S + k[t][:, :, None] * vt[:, None, :]
             o[t] = torch.einsum("hde,hd->he", S, q[t])
+            if skip is not None:
+                o[t] += skip.float()[:, None] * v[t]
         state[slot] = S
     return o.view(T, H * Dv)
 
 
-def gated_rmsnorm(o, w, gate, eps: float, out_dtype):
-    """rmsnorm(o) * w * sigmoid(gate), the row normalised as a whole."""
-    of = o.float()
-    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * w.float()
-    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+def lightning_scan(qkv, H: int, D: int, Dv: int, state, state_slots, cu_q, positions, decay):
+    """Decayed linear attention, token by token: S <- decay_h S + k v^T,
+    o = S^T q with q, k, v = silu of the [q | k | v] columns of ``qkv``. The
+    state [slots, H, D, Dv] (f32) is read at the sequence's slot (zero when
+    the step's first position is 0) and written back. Returns o f32 [T, H Dv]."""
+    a = torch.nn.functional.silu(qkv[:, :2 * H * D + H * Dv].float())
+    return state_scan(a, H, D, Dv, 0, H * D, 2 * H * D, 1, state, state_slots, cu_q, positions,
+                      decay=decay)
+
+
+def gated_rmsnorm(o, w, gate, eps: float, out_dtype, groups: int = 1, silu_first: bool = False):
+    """rmsnorm(o) * w * sigmoid(gate), the row normalised as a whole; with
+    ``silu_first``: rmsnorm(o * silu(gate)) * w (the gate before the norm).
+    ``groups`` > 1 normalises the row in that many equal parts."""
+    of, g = o.float(), gate.float()
+    T, n = of.shape
+    if silu_first:
+        of = of * torch.nn.functional.silu(g)
+    y = of.view(T, groups, n // groups)
+    y = (y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)).view(T, n) * w.float()
+    if not silu_first:
+        y = y * torch.sigmoid(g)
+    return y.to(out_dtype)
 
 
 def moe_route(z, correction, n_groups: int, keep: int, top: int, bias=None,
-              top_softmax: bool = False):
+              top_softmax: bool = False, sigmoid: bool = False, group_rank: int = 1):
     """z f32 [T, E] router logits (+ ``bias`` [E]) -> (expert index int32 [T, top],
     weight f32 [T, top]). Default: scores are softmax(z); experts are chosen by
     score + correction among the ``keep`` best of ``n_groups`` equal groups of
     neighbours (a group's rank is its best choice score); the weights are the
     plain scores. ``top_softmax``: the ``top`` largest logits are chosen and the
-    weights are the softmax over the chosen logits only."""
+    weights are the softmax over the chosen logits only. ``sigmoid``: the scores
+    are sigmoid(z) instead of the softmax. ``group_rank`` n: a group ranks by the
+    sum of its n best choice scores."""
     z = z.float() if bias is None else z.float() + bias.float()
     if top_softmax:
         best = z.topk(top, dim=-1)
         return best.indices.to(torch.int32), torch.softmax(best.values, dim=-1)
-    s = torch.softmax(z, dim=-1)
+    s = torch.sigmoid(z) if sigmoid else torch.softmax(z, dim=-1)
     choice = s if correction is None else s + correction.float()
     if n_groups > 1 and keep < n_groups:
         T, E = s.shape
         per = E // n_groups
-        gs = choice.view(T, n_groups, per).max(-1).values
+        gs = choice.view(T, n_groups, per).topk(min(max(group_rank, 1), per), dim=-1).values.sum(-1)
         kept = gs.topk(keep, dim=-1).indices
         ok = torch.zeros(T, n_groups, dtype=torch.bool, device=z.device).scatter_(1, kept, True)
         choice = choice.masked_fill(~ok.repeat_interleave(per, dim=1), float("-inf"))
@@ -932,3 +979,130 @@ def scalar_rms_norm(x, g: float, eps: float, row_idx=None):
         x = x.index_select(0, row_idx.long())
     xf = x.float()
     return xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * g
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of pre-norm decoders with softmax attention over paged K / V
+# and Mamba-2 layers (models/movinex.py): RMS norm with a weight stored around
+# zero fused with the layer-scaled residual step, per-head q / k preparation
+# (interleaved rotary, weightless RMS norm, query temperature) with the paged
+# append, softmax attention with a sliding window, kept first tokens and score
+# soft-capping, and the Mamba-2 input stage (convolution, step sizes, decays).
+def rms1p_norm(x, w, eps: float, out_dtype, row_idx=None):
+    """x / sqrt(mean(x^2) + eps) * (1 + w) over rows (``row_idx`` gathers first)."""
+    if row_idx is not None:
+        x = x.index_select(0, row_idx.long())
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float())).to(out_dtype)
+
+
+def scaled_add_rms1p(resid, y, ls, nxt, eps: float, out_dtype):
+    """resid (f32, in place) += ls * y per coordinate; returns
+    rms1p_norm(resid; nxt) in ``out_dtype``, or None without ``nxt``."""
+    resid.add_(y.float() * ls.float())
+    return None if nxt is None else rms1p_norm(resid, nxt, eps, out_dtype)
+
+
+def qk_prep_append(u, H: int, G: int, D: int, Dv: int, v_off: int, cos_sin, dims: int, eps: float,
+                   q_temp, positions, k_cache, v_cache, slots, out_dtype):
+    """u [T, >= H D + G D (+ G Dv)]: projected q | k (| v) rows. Per head: the
+    first ``dims`` entries of q and k rotate pairwise (2i with 2i + 1) by the
+    position's angles, then each head's q and k is divided by its root mean
+    square (eps inside the root, no weight); q is multiplied by the position's
+    temperature 1 + coef ln(floor((p + 1) / every) + 1) when ``q_temp`` =
+    (coef, every). k goes to its pages [blocks, BLK, G D]; the value rows - the
+    columns at ``v_off``, or with ``v_off`` < 0 the k columns as projected - go to
+    theirs [blocks, BLK, G Dv] at ``slots`` (-1: padding row). Returns q [T, H D]."""
+    T = u.shape[0]
+    uf = u.float()
+    q = uf[:, :H * D].reshape(T, H, D)
+    k = uf[:, H * D:(H + G) * D].reshape(T, G, D)
+    v = k.reshape(T, G * D) if v_off < 0 else uf[:, v_off:v_off + G * Dv]
+    pos = positions[:T].long()
+    if dims:
+        cs = cos_sin[pos]
+        q, k = rotate_pairs(q, cs, dims), rotate_pairs(k, cs, dims)
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+    if q_temp is not None:
+        coef, every = q_temp
+        steps = torch.div(pos + 1, int(every), rounding_mode="floor").float()
+        q = q * (1.0 + float(coef) * torch.log(steps + 1.0))[:, None, None]
+    sl = slots[:T].long()
+    ok = sl >= 0
+    blk = k_cache.shape[1]
+    k_cache[(sl // blk)[ok], (sl % blk)[ok]] = k.reshape(T, G * D).to(k_cache.dtype)[ok]
+    v_cache[(sl // blk)[ok], (sl % blk)[ok]] = v.to(v_cache.dtype)[ok]
+    return q.reshape(T, H * D).to(out_dtype)
+
+
+def window_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions, scale: float,
+                     softcap: float, window: int, keep_first: int, gate, H: int, G: int, D: int,
+                     Dv: int, out_dtype):
+    """Softmax attention of q [T, H D] over paged K [blocks, BLK, G D] and V
+    [blocks, BLK, G Dv]: score = q . k * scale, soft-capped to cap tanh(score /
+    cap) when ``softcap`` > 0; a query at position p sees key j <= p, and with
+    ``window`` > 0 only if p - j < window or j < keep_first. ``gate`` [T, H Dv]
+    multiplies the output by sigmoid(gate) per entry. Returns [T, H Dv]."""
+    T = q.shape[0]
+    blk = k_cache.shape[1]
+    rep = H // G
+    cu = cu_q.tolist()
+    out = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    qf = q.float().view(T, H, D)
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        L = int(ctx_lens[b])
+        idx = torch.arange(L, device=q.device)
+        tab = block_tables[b].long()
+        kk = k_cache[tab[idx // blk], idx % blk].float().view(L, G, D)
+        vv = v_cache[tab[idx // blk], idx % blk].float().view(L, G, Dv)
+        qpos = positions[q0:q1].long()
+        seen = idx[None, :] <= qpos[:, None]
+        if window > 0:
+            seen &= ((qpos[:, None] - idx[None, :]) < window) | (idx[None, :] < keep_first)
+        for h in range(H):
+            s = qf[q0:q1, h] @ kk[:, h // rep].T * scale
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
+            s = s.masked_fill(~seen, float("-inf"))
+            out[q0:q1, h] = torch.softmax(s, dim=-1) @ vv[:, h // rep]
+    out = out.view(T, H * Dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(out_dtype)
+
+
+def mamba2_prep(u, x_off: int, C: int, dt_off: int, Hh: int, conv_w, conv_b, dt_bias, a_neg, tail,
+                state_slots, cu_q, positions):
+    """The input stage of a Mamba-2 layer over a flat token batch. u [T, W]:
+    the projected row; its columns x_off .. x_off + C pass a causal convolution
+    per channel (weights tap-major [taps, C], the last tap is the current
+    token's; rows before the feed from ``tail[slot]``, zeros before position 0),
+    plus ``conv_b``, then SiLU -> f32 [T, C]. The columns dt_off .. dt_off + Hh
+    give the step sizes dt = softplus(u + dt_bias) and the decays exp(a_neg dt)
+    -> f32 [T, Hh, 2] = (decay, dt)."""
+    T = u.shape[0]
+    taps = conv_w.shape[0]
+    cu = cu_q.tolist()
+    xin = u[:, x_off:x_off + C].float()
+    y = torch.zeros(T, C, dtype=torch.float32, device=u.device)
+    w = conv_w.float()
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        if taps > 1:
+            old = torch.zeros_like(tail[0]) if int(positions[q0]) == 0 else \
+                tail[int(state_slots[b])]
+            rows = torch.cat([old.float(), xin[q0:q1]])
+        else:
+            rows = xin[q0:q1]
+        n = q1 - q0
+        for j in range(taps):
+            y[q0:q1] += rows[j:j + n] * w[j]
+    y = torch.nn.functional.silu(y + conv_b.float())
+    dt = torch.nn.functional.softplus(u[:, dt_off:dt_off + Hh].float() + dt_bias.float())
+    return y, torch.stack([torch.exp(a_neg.float() * dt), dt], dim=-1).contiguous()

@@ -248,60 +248,117 @@ def lightning_scan(qkv: torch.Tensor, H: int, D: int, Dv: int, state: torch.Tens
     _i32c(state_slots, "state_slots"); _i32c(cu_q, "cu_q"); _i32c(positions, "positions")
     B = state_slots.numel()
     assert cu_q.numel() == B + 1
-    o = torch.empty(T, H * Dv, dtype=torch.float32, device=qkv.device)
+    if not T:
+        return torch.empty(0, H * Dv, dtype=torch.float32, device=qkv.device)
+    # SiLU of q | k | v once, in f32 (every column block of a head shares q and k)
+    n = 2 * H * D + H * Dv
+    act = torch.empty(T, n, dtype=torch.float32, device=qkv.device)
+    check(kernels().loqa_lightning_prep(ptr(qkv), _dt(qkv), qkv.stride(0), T, n, ptr(act),
+                                        stream_ptr(qkv)), "lightning_prep")
+    return state_scan(act, H, D, Dv, 0, H * D, 2 * H * D, 1, state, state_slots, cu_q, positions,
+                      decay=decay)
+
+
+def state_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int,
+               hpg: int, state: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+               positions: torch.Tensor, decay: torch.Tensor | None = None,
+               tok: torch.Tensor | None = None, skip: torch.Tensor | None = None) -> torch.Tensor:
+    """The linear recurrence with a carried matrix state that decayed linear
+    attention and Mamba-2 layers share, per sequence and head, token by token
+    in f32:  S <- a S + k (c v)^T,  o = S^T q + skip_h v,  with a = ``decay[h]``
+    or per token ``tok[t, h, 0]`` and c = 1 or ``tok[t, h, 1]``. ``act`` f32
+    [T, W]: head h reads q at ``q_off + (h // hpg) D``, k at ``k_off + (h // hpg)
+    D`` and v at ``v_off + h Dv``. ``state`` [slots, H, D, Dv] f32 carries S
+    between steps (zero when the step's first position is 0). One kernel and
+    one order of operations for prompt portions and single tokens."""
+    if not act.is_cuda:
+        return ref.state_scan(act, H, D, Dv, q_off, k_off, v_off, hpg, state, state_slots, cu_q,
+                              positions, decay, tok, skip)
+    T, W = act.shape
+    _f32c(act, "act"); _f32c(state, "state")
+    assert state.shape[1:] == (H, D, Dv) and hpg >= 1 and H % hpg == 0
+    G = H // hpg
+    assert min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + G * D <= W and v_off + H * Dv <= W
+    assert (decay is None) != (tok is None)
+    if decay is not None:
+        _f32c(decay, "decay")
+        assert decay.numel() == H
+    else:
+        _f32c(tok, "tok")
+        assert tok.shape == (T, H, 2)
+    if skip is not None:
+        _f32c(skip, "skip")
+        assert skip.numel() == H
+    _i32c(state_slots, "state_slots"); _i32c(cu_q, "cu_q"); _i32c(positions, "positions")
+    B = state_slots.numel()
+    assert cu_q.numel() == B + 1 and positions.numel() >= T
+    o = torch.empty(T, H * Dv, dtype=torch.float32, device=act.device)
     if T:
-        # SiLU of q | k | v once, in f32 (every column block of a head shares q and k)
-        n = 2 * H * D + H * Dv
-        act = torch.empty(T, n, dtype=torch.float32, device=qkv.device)
-        k, st = kernels(), stream_ptr(qkv)
-        check(k.loqa_lightning_prep(ptr(qkv), _dt(qkv), qkv.stride(0), T, n, ptr(act), st),
-              "lightning_prep")
-        check(k.loqa_lightning_scan(ptr(act), n, H, D, Dv, ptr(state), state.shape[0],
-                                    ptr(state_slots), ptr(cu_q), ptr(positions), ptr(decay), ptr(o),
-                                    B, T, st), "lightning_scan")
+        check(kernels().loqa_state_scan(ptr(act), W, H, D, Dv, q_off, k_off, v_off, hpg, ptr(state),
+                                        state.shape[0], ptr(state_slots), ptr(cu_q), ptr(positions),
+                                        ptr(decay), ptr(tok), ptr(skip), ptr(o), B, T,
+                                        stream_ptr(act)), "state_scan")
     return o
 
 
 def gated_rmsnorm(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, eps: float,
-                  out_dtype) -> torch.Tensor:
-    """y = rmsnorm(o) * w * sigmoid(gate) over whole rows of o f32 [T, n];
-    ``gate`` [T, n] may be a column slice of a wider projection."""
+                  out_dtype, groups: int = 1, silu_first: bool = False) -> torch.Tensor:
+    """y = rmsnorm(o) * w * sigmoid(gate) over whole rows of o f32 [T, n], or
+    with ``silu_first`` y = rmsnorm(o * silu(gate)) * w (the gate before the
+    norm); ``groups`` > 1 normalises a row in that many equal parts, each by
+    its own root mean square. ``gate`` [T, n] may be a column slice of a wider
+    projection."""
     if not o.is_cuda:
-        return ref.gated_rmsnorm(o, w, gate, eps, out_dtype)
+        return ref.gated_rmsnorm(o, w, gate, eps, out_dtype, groups, silu_first)
     _f32c(o, "o"); _f32c(w, "w")
     T, n = o.shape
     assert gate.shape == (T, n) and gate.stride(1) == 1 and w.numel() == n
+    assert groups >= 1 and n % groups == 0
     y = torch.empty(T, n, dtype=out_dtype, device=o.device)
     if T:
         check(kernels().loqa_gated_rmsnorm(ptr(o), ptr(w), ptr(gate), _dt(gate), gate.stride(0), eps,
-                                           ptr(y), _dt(y), T, n, stream_ptr(o)), "gated_rmsnorm")
+                                           ptr(y), _dt(y), T, n, groups, int(silu_first),
+                                           stream_ptr(o)), "gated_rmsnorm")
+    return y
+
+
+_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+
+def act_mul_any(x: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """[gate | up] -> act(gate) * up for bf16 or f32 activations; ``act`` is
+    "silu" or "gelu_tanh" (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))))."""
+    if not x.is_cuda:
+        return ref.silu_mul(x) if act == "silu" else ref.act_mul(x, act)
+    assert x.dim() == 2 and x.is_contiguous() and x.shape[1] % 2 == 0
+    T, F2 = x.shape
+    y = torch.empty(T, F2 // 2, dtype=x.dtype, device=x.device)
+    if T:
+        check(kernels().loqa_act_mul_any(ptr(x), _dt(x), T, F2 // 2, _ACTS[act], ptr(y),
+                                         stream_ptr(x)), "act_mul_any")
     return y
 
 
 def silu_mul_any(x: torch.Tensor) -> torch.Tensor:
     """[gate | up] -> silu(gate) * up for bf16 or f32 activations."""
-    if not x.is_cuda:
-        return ref.silu_mul(x)
-    assert x.dim() == 2 and x.is_contiguous() and x.shape[1] % 2 == 0
-    T, F2 = x.shape
-    y = torch.empty(T, F2 // 2, dtype=x.dtype, device=x.device)
-    if T:
-        check(kernels().loqa_silu_mul_any(ptr(x), _dt(x), T, F2 // 2, ptr(y), stream_ptr(x)),
-              "silu_mul_any")
-    return y
+    return act_mul_any(x, "silu")
 
 
 def moe_route(z: torch.Tensor, correction: torch.Tensor | None, n_groups: int, keep: int,
-              top: int, bias: torch.Tensor | None = None, top_softmax: bool = False
-              ) -> tuple[torch.Tensor, torch.Tensor]:
+              top: int, bias: torch.Tensor | None = None, top_softmax: bool = False,
+              sigmoid: bool = False, group_rank: int = 1) -> tuple[torch.Tensor, torch.Tensor]:
     """Router decisions from f32 logits z [T, E] (+ ``bias`` [E]). Default:
     softmax scores, choice by score + ``correction`` limited to the ``keep``
     best of ``n_groups`` groups of neighbouring experts, weights = the plain
     scores (not renormalised). ``top_softmax``: the ``top`` largest logits are
-    chosen and weighed by the softmax over the chosen logits only.
+    chosen and weighed by the softmax over the chosen logits only. ``sigmoid``:
+    the scores are sigmoid(z) instead of the softmax. ``group_rank`` n: a group
+    ranks by the sum of its n best choice scores instead of its best one.
     Returns (idx int32 [T, top], weight f32 [T, top])."""
     if not z.is_cuda:
-        return ref.moe_route(z, correction, n_groups, keep, top, bias, top_softmax)
+        return ref.moe_route(z, correction, n_groups, keep, top, bias, top_softmax, sigmoid,
+                             group_rank)
+    assert not (top_softmax and sigmoid)
     _f32c(z, "z")
     T, E = z.shape
     assert E % max(1, n_groups) == 0 and 0 < top <= E and E <= 1024
@@ -312,9 +369,11 @@ def moe_route(z: torch.Tensor, correction: torch.Tensor | None, n_groups: int, k
     idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
     wt = torch.empty(T, top, dtype=torch.float32, device=z.device)
     if T:
-        check(kernels().loqa_moe_route(ptr(z), ptr(correction), ptr(bias), int(top_softmax), E,
-                                       max(1, n_groups), min(keep, max(1, n_groups)), top, ptr(idx),
-                                       ptr(wt), T, stream_ptr(z)), "moe_route")
+        check(kernels().loqa_moe_route(ptr(z), ptr(correction), ptr(bias),
+                                       1 if top_softmax else (2 if sigmoid else 0), E,
+                                       max(1, n_groups), min(keep, max(1, n_groups)),
+                                       max(1, group_rank), top, ptr(idx), ptr(wt), T,
+                                       stream_ptr(z)), "moe_route")
     return idx, wt
 
 
@@ -544,3 +603,171 @@ def scalar_rms_norm(x: torch.Tensor, g: float, eps: float, row_idx: torch.Tensor
         check(kernels().loqa_scalar_rms_norm(ptr(x), ptr(row_idx), float(g), float(eps), ptr(y), rows,
                                              d, stream_ptr(x)), "scalar_rms_norm")
     return y
+
+
+# ---------------------------------------------------------------------------
+# Pre-norm RMS norm with a weight stored around zero and layer scale on the
+# residual step, q / k preparation with paged append, softmax attention with a
+# sliding window / kept first tokens / soft-capping over paged K / V, and the
+# Mamba-2 input stage (csrc/kernels/norm_rms1p.hip, attn_window.hip, mamba2.hip)
+def rms1p_norm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype,
+               row_idx: torch.Tensor | None = None) -> torch.Tensor:
+    """y = x / sqrt(mean(x^2) + eps) * (1 + w) over rows of x f32 [rows, d];
+    ``row_idx`` (int64) gathers rows in the same launch."""
+    if not x.is_cuda:
+        return ref.rms1p_norm(x, w, eps, out_dtype, row_idx)
+    _f32c(x, "x"); _f32c(w, "w")
+    d = x.shape[1]
+    assert w.numel() == d
+    rows = x.shape[0] if row_idx is None else row_idx.numel()
+    if row_idx is not None:
+        assert row_idx.dtype == torch.int64 and row_idx.is_contiguous()
+    y = torch.empty(rows, d, dtype=out_dtype, device=x.device)
+    if rows:
+        check(kernels().loqa_rms1p_norm(ptr(x), ptr(row_idx), ptr(w), float(eps), ptr(y), _dt(y),
+                                        rows, d, stream_ptr(x)), "rms1p_norm")
+    return y
+
+
+def scaled_add_rms1p(resid: torch.Tensor, y: torch.Tensor, ls: torch.Tensor,
+                     nxt: torch.Tensor | None, eps: float, out_dtype) -> torch.Tensor | None:
+    """The fused residual step of a pre-norm layer with layer scale: resid (f32,
+    in place) += ls * y per coordinate, and in the same launch the next
+    sublayer's input h = resid / rms(resid) * (1 + nxt) (None: no h)."""
+    if not resid.is_cuda:
+        return ref.scaled_add_rms1p(resid, y, ls, nxt, eps, out_dtype)
+    _f32c(resid, "resid"); _f32c(ls, "ls")
+    assert y.shape == resid.shape and y.is_contiguous()
+    rows, d = resid.shape
+    assert ls.numel() == d
+    h = None
+    if nxt is not None:
+        _f32c(nxt, "nxt")
+        assert nxt.numel() == d
+        h = torch.empty(rows, d, dtype=out_dtype, device=resid.device)
+    if rows:
+        check(kernels().loqa_scaled_add_rms1p(ptr(resid), ptr(y), _dt(y), ptr(ls), ptr(nxt),
+                                              float(eps), ptr(h), _dt(h) if h is not None else 0,
+                                              rows, d, stream_ptr(resid)), "scaled_add_rms1p")
+    return h
+
+
+def qk_prep_append(u: torch.Tensor, H: int, G: int, D: int, Dv: int, v_off: int,
+                   cos_sin: torch.Tensor | None, dims: int, eps: float, q_temp: tuple | None,
+                   positions: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   slots: torch.Tensor, out_dtype) -> torch.Tensor:
+    """One launch between the fused q | k (| v) projection u [T, W] and
+    attention: per head the first ``dims`` entries of q and k rotate pairwise
+    (interleaved layout, table ``cos_sin`` [positions, dims / 2, 2]), then q and
+    k are divided by their root mean square over the head (no weight), q is
+    multiplied by the position's temperature 1 + coef ln(floor((p + 1) / every)
+    + 1) (``q_temp`` = (coef, every) or None); k goes to its pages [blocks, BLK,
+    G D] and the value rows - the columns at ``v_off``, or with ``v_off`` < 0
+    the k columns as projected - to theirs [blocks, BLK, G Dv]. Returns q
+    [T, H D]. Statistics, angles and the temperature are f32."""
+    if not u.is_cuda:
+        return ref.qk_prep_append(u, H, G, D, Dv, v_off, cos_sin, dims, eps, q_temp, positions,
+                                  k_cache, v_cache, slots, out_dtype)
+    T, W = u.shape
+    assert u.stride(1) == 1 and (H + G) * D <= W
+    assert v_off < 0 and Dv == D or v_off >= (H + G) * D and v_off + G * Dv <= W
+    assert dims % 2 == 0 and 0 <= dims <= D
+    if dims:
+        _f32c(cos_sin, "cos_sin")
+        assert cos_sin.shape[1] * 2 == dims
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert k_cache.dtype == v_cache.dtype == out_dtype == u.dtype
+    assert k_cache.shape[2] == G * D and v_cache.shape == (*k_cache.shape[:2], G * Dv)
+    _i32c(positions, "positions"); _i32c(slots, "slots")
+    assert positions.numel() >= T and slots.numel() >= T
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 1)
+    q = torch.empty(T, H * D, dtype=out_dtype, device=u.device)
+    if T:
+        check(kernels().loqa_qk_prep_append(
+            ptr(u), _dt(u), u.stride(0), H, G, D, Dv, int(v_off), ptr(cos_sin) if dims else None,
+            cos_sin.shape[0] if dims else 0, dims, float(eps), coef, every, ptr(positions),
+            ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0], ptr(slots), ptr(q), T,
+            stream_ptr(u)), "qk_prep_append")
+    return q
+
+
+WINDOW_MFMA_D = (64, 128)         # head sizes the matrix-core form is built for
+
+
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     cu_q: torch.Tensor, ctx_lens: torch.Tensor, block_tables: torch.Tensor,
+                     positions: torch.Tensor, scale: float, softcap: float, window: int,
+                     keep_first: int, gate: torch.Tensor | None, H: int, G: int, D: int, Dv: int,
+                     max_q: int = 0, matrix_cores: bool | None = None) -> torch.Tensor:
+    """Softmax attention over paged K [blocks, BLK, G D] and V [blocks, BLK,
+    G Dv] (query head h reads key/value head h // (H / G)): score = q . k *
+    scale, soft-capped to cap tanh(score / cap) when ``softcap`` > 0; a query at
+    position p sees key j <= p, with ``window`` > 0 only if p - j < window or
+    j < keep_first (kept keys keep their own positions). ``gate`` [T, H Dv] (may
+    be a column slice) multiplies the output by sigmoid(gate) per entry. q
+    [T, H D] -> [T, H Dv]. Rows find their sequence through ``cu_q`` and their
+    keys through the block table, so prompt portions, decode tokens and mixed
+    batches are one launch. Scores, softmax and accumulators are f32."""
+    if not q.is_cuda:
+        return ref.window_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions,
+                                    scale, softcap, window, keep_first, gate, H, G, D, Dv, q.dtype)
+    T = q.shape[0]
+    assert q.is_contiguous() and q.shape[1] == H * D and H % G == 0
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert k_cache.shape[2] == G * D and k_cache.dtype == v_cache.dtype == q.dtype
+    assert v_cache.shape == (*k_cache.shape[:2], G * Dv)
+    assert D <= 512 and Dv <= 512 and window >= 0 and keep_first >= 0 and softcap >= 0
+    _i32c(cu_q, "cu_q"); _i32c(ctx_lens, "ctx_lens"); _i32c(block_tables, "block_tables")
+    _i32c(positions, "positions")
+    B = ctx_lens.numel()
+    assert cu_q.numel() == B + 1 and block_tables.shape[0] == B and positions.numel() >= T
+    gs = 0
+    if gate is not None:
+        assert gate.shape == (T, H * Dv) and gate.stride(1) == 1 and gate.dtype == q.dtype
+        gs = gate.stride(0)
+    o = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    if matrix_cores is None:
+        matrix_cores = max_q >= 16
+    mfma = bool(matrix_cores) and q.dtype == torch.bfloat16 and D in WINDOW_MFMA_D \
+        and Dv in WINDOW_MFMA_D and k_cache.shape[1] % 8 == 0
+    if T:
+        check(kernels().loqa_window_attention(
+            ptr(q), _dt(q), ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0],
+            ptr(cu_q), ptr(ctx_lens), ptr(block_tables), block_tables.shape[1], ptr(positions),
+            ptr(gate), gs, float(scale), float(softcap), int(window), int(keep_first), B, T, H, G,
+            D, Dv, int(max_q), int(mfma), ptr(o), stream_ptr(q)), "window_attention")
+    return o
+
+
+def mamba2_prep(u: torch.Tensor, x_off: int, C: int, dt_off: int, Hh: int, conv_w: torch.Tensor,
+                conv_b: torch.Tensor, dt_bias: torch.Tensor, a_neg: torch.Tensor,
+                tail: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+                positions: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The input stage of a Mamba-2 layer, one launch over a flat token batch:
+    the columns x_off .. x_off + C of the projected rows u [T, W] pass a causal
+    convolution per channel (f32 weights tap-major [taps, C], last tap = the
+    current token; the rows before a feed from ``tail[slot]`` f32 [slots, taps -
+    1, C], zeros before position 0) plus ``conv_b``, then SiLU -> f32 [T, C];
+    the columns dt_off .. dt_off + Hh give dt = softplus(u + dt_bias) and the
+    decay exp(a_neg dt) per head -> f32 [T, Hh, 2] = (decay, dt). ``tail`` is
+    not written here (:func:`seq_state_save` does, after every reader)."""
+    if not u.is_cuda:
+        return ref.mamba2_prep(u, x_off, C, dt_off, Hh, conv_w, conv_b, dt_bias, a_neg, tail,
+                               state_slots, cu_q, positions)
+    T, W = u.shape
+    taps = conv_w.shape[0]
+    assert u.stride(1) == 1 and x_off + C <= W and dt_off + Hh <= W and conv_w.shape == (taps, C)
+    for t, name, n in ((conv_w, "conv_w", taps * C), (conv_b, "conv_b", C),
+                       (dt_bias, "dt_bias", Hh), (a_neg, "a_neg", Hh), (tail, "tail", None)):
+        _f32c(t, name)
+        assert n is None or t.numel() == n
+    assert tail.shape[1:] == (taps - 1, C)
+    B = _seq_args(state_slots, cu_q, positions, T)
+    xbc = torch.empty(T, C, dtype=torch.float32, device=u.device)
+    tok = torch.empty(T, Hh, 2, dtype=torch.float32, device=u.device)
+    if T:
+        check(kernels().loqa_mamba2_prep(
+            ptr(u), _dt(u), u.stride(0), x_off, C, dt_off, Hh, ptr(conv_w), taps, ptr(conv_b),
+            ptr(dt_bias), ptr(a_neg), ptr(tail), tail.shape[0], ptr(state_slots), ptr(cu_q),
+            ptr(positions), B, T, ptr(xbc), ptr(tok), stream_ptr(u)), "mamba2_prep")
+    return xbc, tok
