@@ -5,9 +5,11 @@
 //   outputs; choice = score + correction; router outputs form `groups` equal
 //   groups of neighbours, a group ranks by its best choice score and only the
 //   `keep` best groups stay eligible (the others count as -inf); the `top`
-//   best eligible choices are taken; the weights are the plain scores. With
-//   `top_softmax` the choice is by the logit itself (+ bias) and the weights
-//   are the softmax over the chosen logits only.
+//   best eligible choices are taken; the weights are the plain scores. Mode 1:
+//   the choice is by the logit itself (+ bias) and the weights are the softmax
+//   over the chosen logits only. Mode 2: scores = sigmoid(z) instead of the
+//   softmax. With `grank` n > 1 a group ranks by the sum of its n best choice
+//   scores.
 // moe_plan_kernel (one workgroup): (token, k) pairs bucketed by expert without
 //   a host round trip: offsets[E + 2], perm[P] (pair ids in expert order; the
 //   identity bucket E last), pos[P] (where each pair sits).
@@ -34,8 +36,9 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 
 __global__ __launch_bounds__(64) void moe_route_kernel(
     const float* __restrict__ z, const float* __restrict__ corr, const float* __restrict__ bias,
-    int top_softmax, int E, int G, int keep, int top, int* __restrict__ idx,
+    int mode, int E, int G, int keep, int grank, int top, int* __restrict__ idx,
     float* __restrict__ wt) {
+  const int top_softmax = mode == 1;
   __shared__ float sc[MOE_MAX_E], ch[MOE_MAX_E], gs[MOE_MAX_E];
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (size_t)t * E;
@@ -48,12 +51,12 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
   mx = wave_max(mx);
   float sum = 0.f;
   for (int e = lane; e < E; e += 64) {
-    const float v = expf(gs[e] - mx);
+    const float v = mode == 2 ? sigmoid_f(gs[e]) : expf(gs[e] - mx);
     sc[e] = v;
     sum += v;
   }
   sum = wave_sum(sum);
-  const float inv = 1.f / sum;
+  const float inv = mode == 2 ? 1.f : 1.f / sum;
   for (int e = lane; e < E; e += 64) {
     if (top_softmax) { ch[e] = gs[e]; continue; }      // scores stay unnormalised: see below
     const float s = sc[e] * inv;
@@ -65,7 +68,28 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
     const int per = E / G;
     for (int g = lane; g < G; g += 64) {
       float b = -INFINITY;
-      for (int j = 0; j < per; ++j) b = fmaxf(b, ch[g * per + j]);
+      if (grank <= 1) {
+        for (int j = 0; j < per; ++j) b = fmaxf(b, ch[g * per + j]);
+      } else {
+        // the sum of the group's n best: n passes, each taking the largest entry
+        // below the previous one (by value, then index)
+        float pv = INFINITY;
+        int pi = -1;
+        b = 0.f;
+        for (int n = 0; n < min(grank, per); ++n) {
+          float bv = -INFINITY;
+          int bi = -1;
+          for (int j = 0; j < per; ++j) {
+            const float v = ch[g * per + j];
+            const bool below = v < pv || (v == pv && j > pi);
+            if (below && (bi < 0 || v > bv)) { bv = v; bi = j; }
+          }
+          if (bi < 0) break;
+          b += bv;
+          pv = bv;
+          pi = bi;
+        }
+      }
       gs[g] = b;
     }
     __syncthreads();
@@ -461,35 +485,45 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void silu_mul_any_kernel(const T* __restrict__ x, int F,
-                                                           T* __restrict__ y) {
-  const size_t r = blockIdx.x;
-  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < F; c += gridDim.y * blockDim.x)
-    Act<T>::st(y + r * F + c,
-               silu_f(Act<T>::ld(x + r * 2 * F + c)) * Act<T>::ld(x + r * 2 * F + F + c));
+// 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-extern "C" int loqa_silu_mul_any(const void* x, int dt, int T, int F, void* y, hipStream_t st) {
+// ACT 0: SiLU, 1: the tanh form of GELU
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void act_mul_any_kernel(const T* __restrict__ x, int F,
+                                                          T* __restrict__ y) {
+  const size_t r = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < F; c += gridDim.y * blockDim.x) {
+    const float g = Act<T>::ld(x + r * 2 * F + c);
+    Act<T>::st(y + r * F + c, (ACT == 1 ? gelu_tanh_f(g) : silu_f(g)) * Act<T>::ld(x + r * 2 * F + F + c));
+  }
+}
+
+extern "C" int loqa_act_mul_any(const void* x, int dt, int T, int F, int act, void* y,
+                                hipStream_t st) {
   if (T <= 0) return 0;
+  if (act < 0 || act > 1) return (int)hipErrorInvalidValue;
   const dim3 grid(T, T >= 512 ? 1 : (F + 255) / 256);
-  if (dt == 0)
-    hipLaunchKernelGGL(silu_mul_any_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, F,
-                       (bf16_t*)y);
-  else
-    hipLaunchKernelGGL(silu_mul_any_kernel<float>, grid, dim3(256), 0, st, (const float*)x, F,
-                       (float*)y);
+#define GO(TT, A)                                                                             \
+  hipLaunchKernelGGL((act_mul_any_kernel<TT, A>), grid, dim3(256), 0, st, (const TT*)x, F, (TT*)y)
+  if (dt == 0 && act == 0) GO(bf16_t, 0);
+  else if (dt == 0) GO(bf16_t, 1);
+  else if (act == 0) GO(float, 0);
+  else GO(float, 1);
+#undef GO
   return (int)hipGetLastError();
 }
 
-extern "C" int loqa_moe_route(const void* z, const void* corr, const void* bias, int top_softmax,
-                              int E, int G, int keep, int top, void* idx, void* wt, int T,
-                              hipStream_t st) {
+extern "C" int loqa_moe_route(const void* z, const void* corr, const void* bias, int mode,
+                              int E, int G, int keep, int grank, int top, void* idx, void* wt,
+                              int T, hipStream_t st) {
   if (T <= 0) return 0;
-  if (E > MOE_MAX_E || E <= 0 || G <= 0 || E % G || top <= 0 || top > E)
+  if (E > MOE_MAX_E || E <= 0 || G <= 0 || E % G || top <= 0 || top > E || mode < 0 || mode > 2)
     return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(64), 0, st, (const float*)z, (const float*)corr,
-                     (const float*)bias, top_softmax, E, G, keep, top, (int*)idx, (float*)wt);
+                     (const float*)bias, mode, E, G, keep, grank, top, (int*)idx, (float*)wt);
   return (int)hipGetLastError();
 }
 
