@@ -482,7 +482,6 @@ __global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnPar
 
 int window_attention_mfma(const WinAttnParams& p, int max_q, hipStream_t st) {
   if (max_q <= 0) return 0;
-  if (p.gate && (p.gate_ld % 4 || ((size_t)p.gate & 7))) return (int)hipErrorInvalidValue;
   const dim3 grid((max_q + WM_WAVES * 32 - 1) / (WM_WAVES * 32), p.H, p.B);
 #define GO(A, C)                                                                              \
   if (p.D == A && p.Dv == C) {                                                                \
@@ -529,7 +528,9 @@ extern "C" int loqa_window_attention(const void* q, int dt, const void* kc, cons
   p.max_blocks = max_blocks; p.pos = (const int*)pos; p.gate = gate; p.gate_ld = gate_ld;
   p.scale = scale; p.cap = cap; p.window = window; p.keep_first = keep_first;
   p.B = B; p.T = T; p.H = H; p.G = G; p.D = D; p.Dv = Dv; p.o = o;
-  if (mfma && dt == 0 && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) && blk % 8 == 0)
+  // the matrix-core form reads the gate in 8-byte runs
+  const bool gate_ok = !gate || (gate_ld % 4 == 0 && ((size_t)gate & 7) == 0);
+  if (mfma && dt == 0 && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) && gate_ok)
     return window_attention_mfma(p, max_q, st);
   const int rep = H / G;
   const int nv = Dv <= 128 ? 2 : 8;

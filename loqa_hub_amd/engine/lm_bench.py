@@ -3,9 +3,10 @@ engine's step function, at layer sizes that resemble real models (random
 weights, synthetic tokens): ``python bench.py --lm-bench``.
 
 For each size a Pipizen stack (latent attention / lightning mixers, dense and
-mixture-of-experts feed-forwards) and a Sodonex stack (chunked sigmoid
-attention with token shift and short convolutions, squared-relu experts) run
-beside a Llama stack of the same width, depth, head count and feed-forward
+mixture-of-experts feed-forwards), a Sodonex stack (chunked sigmoid attention
+with token shift and short convolutions, squared-relu experts) and a Movinex
+stack (a Mamba-2 layer, full and sliding-window softmax attention, GeGLU and
+sigmoid-routed experts) run beside a Llama stack of the same width, depth, head count and feed-forward
 width - the framework's plain decoder. Measured per family:
 
 * prefill: one prompt of ``P`` tokens through ``LLMEngine.step_logits``;
@@ -24,8 +25,9 @@ import numpy as np
 import torch
 
 from ..models.configs import (ChunkAttnConfig, FeedForwardConfig, HybridLayerConfig,
-                              LatentAttnConfig, LightningConfig, LlamaConfig, PipizenConfig,
-                              RotaryConfig, SodonexConfig)
+                              LatentAttnConfig, LightningConfig, LlamaConfig, LoopConfig,
+                              Mamba2Config, MovinexConfig, PipizenConfig, RotaryConfig,
+                              SodonexConfig, SoftmaxAttnConfig)
 
 SIZES = {
     # name: (width, layers, heads, head_dim, rot_dim, kv_rank, ff, experts, expert_ff, top)
@@ -62,6 +64,29 @@ def sodonex_stack(name: str, vocab: int = 32000, chunk: int = 768) -> SodonexCon
     mlp = FeedForwardConfig("moe", eff, E, 0, top, act="relu2", router="softmax_top")
     return SodonexConfig(f"sodonex-{name}", vocab, d, 1e-6, 0.5, 1.0,
                          tuple(HybridLayerConfig("attention", mixer, mlp) for _ in range(n)))
+
+
+def movinex_stack(name: str, vocab: int = 32000, window: int = 1024) -> MovinexConfig:
+    """Four layers: a Mamba-2 layer (inner width 2 x width, 64 channels per
+    head, state 128) with a dense GeGLU, a full-causal attention layer with
+    biases and query temperature, and two sliding-window layers (keys double as
+    values, rotary, soft-capping, output gate), the three attention layers with
+    sigmoid-routed experts; 4 query heads per key/value head. Layers 1 - 2 are
+    entered through the [x ; embedding] projection of a repeated stretch
+    (one pass, so the stack stays four layer runs deep)."""
+    d, n, H, D, Dr, _, ff, E, eff, top = SIZES[name]
+    G = max(1, H // 4)
+    mamba = Mamba2Config(max(1, 2 * d // 64), min(64, 2 * d), 128 if d >= 512 else 8, 1, 4, 1)
+    full = SoftmaxAttnConfig(H, G, D, D, D ** -0.5, bias=True, q_temp=(0.1, 256))
+    local = SoftmaxAttnConfig(H, G, D, D, D ** -0.5, values_from_keys=True, gate=True,
+                              rot=RotaryConfig(Dr, 10000.0), softcap=30.0, window=window,
+                              keep_first=4)
+    moe = FeedForwardConfig("moe", eff, E, 0, top, 4, 2, router="sigmoid", group_rank=2)
+    layers = [HybridLayerConfig("mamba2", mamba, FeedForwardConfig("dense", ff, act="geglu")),
+              HybridLayerConfig("attention", full, moe)]
+    layers += [HybridLayerConfig("attention_2", local, moe) for _ in range(max(0, n - 2))]
+    return MovinexConfig(f"movinex-{name}", vocab, d, 1e-6, 1.0, tuple(layers),
+                         LoopConfig(1, min(3, len(layers)), 1))
 
 
 def llama_stack(name: str, vocab: int = 32000) -> LlamaConfig:
@@ -131,7 +156,8 @@ def run(args) -> int:
         else torch.device("cpu")
     sizes = [s for s in args.lm_sizes.split(",") if s]
     for name in sizes:
-        fams = {"pipizen": pipizen_stack, "sodonex": sodonex_stack, "llama": llama_stack}
+        fams = {"pipizen": pipizen_stack, "sodonex": sodonex_stack, "movinex": movinex_stack,
+                "llama": llama_stack}
         for fam in [f for f in args.lm_families.split(",") if f]:
             cfg = fams[fam](name)
             if dev.type == "cpu":      # plumbing run: tiny stacks

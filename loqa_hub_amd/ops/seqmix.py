@@ -729,7 +729,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if matrix_cores is None:
         matrix_cores = max_q >= 16
     mfma = bool(matrix_cores) and q.dtype == torch.bfloat16 and D in WINDOW_MFMA_D \
-        and Dv in WINDOW_MFMA_D and k_cache.shape[1] % 8 == 0
+        and Dv in WINDOW_MFMA_D
     if T:
         check(kernels().loqa_window_attention(
             ptr(q), _dt(q), ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0],
