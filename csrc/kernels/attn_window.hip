@@ -23,28 +23,59 @@
 // short feeds and the exact f32 mode): a workgroup per (token, key/value head)
 // serves REP query heads of the group at once, so K and V are read once per
 // group. The visible keys go in 64-key windows aligned to multiples of 64
-// positions, one per wave in turn (window index modulo the wave count): scores
+// positions, one per wave in turn (window index modulo the wave count; 16 waves
+// when the launch has few workgroups, else 4): scores
 // with a lane per key, an online softmax per head across the wave, values with
 // a lane per output column. The waves' partial (max, sum, accumulator) triples
 // merge through LDS in wave order. Which windows a wave takes and the order of
-// every sum depend only on the query's position, never on the batch.
+// every sum depend only on the query's position and the wave count. When a
+// step has few rows and long contexts the windows are also dealt out to several
+// workgroups per row, whose partial triples a small combine launch merges.
 //
 // window_attn_mfma_kernel (bf16, D and Dv in {64, 128}; prompt portions): a
-// workgroup per (128 query rows of one sequence, query head); each wave owns 32
-// rows. K and V tiles of 64 keys are gathered from the pages into LDS for all
+// workgroup per (64 or 128 query rows of one sequence, query head); each wave
+// owns 32 rows. The block-table entries of the key range go to LDS once. K and V tiles of 64 keys are gathered from the pages into LDS for all
 // waves (the next tile's 16-byte chunks already in flight in registers);
 // S^T = K Q^T and O^T += V^T P^T run on v_mfma_f32_32x32x16_bf16 with the query
 // on the MFMA lane, so the online softmax is in-register. Tiles that lie wholly
 // between the kept first tokens and the rows' windows are skipped.
 #include "seqmix.h"
 
-#define WA_NW 4                      // waves of the keys form
-
 struct WinAttnParams {
   const void* q; const void* kc; const void* vc; int blk; long cache_rows;
   const int* cu_q; const int* ctx; const int* bt; int max_blocks; const int* pos;
   const void* gate; long gate_ld; float scale, cap; int window, keep_first;
   int B, T, H, G, D, Dv; void* o;
+  int ns; float* part;               // key splits over workgroups and their partial results
+};
+
+// K / V pages (and the block table) are read through pointers in the global
+// address space: a load through a generic pointer counts against the LDS
+// counter as well, so every wait for an LDS read would also wait for the cache
+// rows in flight and the loads would run one after the other.
+#define WA_GLOBAL __attribute__((address_space(1)))
+typedef unsigned wa_u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct GAct;
+template <> struct GAct<bf16_t> {
+  static constexpr int N = 8;                     // elements of a 16-byte run
+  static __device__ __forceinline__ float ld(const WA_GLOBAL bf16_t* p) { return bf2f(*p); }
+  static __device__ __forceinline__ void ldv(const WA_GLOBAL bf16_t* p, float* f) {
+    const wa_u32x4 v = *reinterpret_cast<const WA_GLOBAL wa_u32x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(v[i] << 16);
+      f[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+  }
+};
+template <> struct GAct<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ float ld(const WA_GLOBAL float* p) { return *p; }
+  static __device__ __forceinline__ void ldv(const WA_GLOBAL float* p, float* f) {
+    const float4v v = *reinterpret_cast<const WA_GLOBAL float4v*>(p);
+    f[0] = v[0]; f[1] = v[1]; f[2] = v[2]; f[3] = v[3];
+  }
 };
 
 __device__ __forceinline__ int wa_seq_of_row(const int* __restrict__ cu_q, int B, int t) {
@@ -117,35 +148,23 @@ __global__ __launch_bounds__(256) void qk_prep_append_kernel(
 }
 
 // ------------------------------------------------------------ few rows, many keys
-template <typename T> struct WaVec;
-template <> struct WaVec<bf16_t> {
-  static constexpr int N = 8;
-  static __device__ __forceinline__ void ld(const bf16_t* p, float* f) {
-    unpack8(*reinterpret_cast<const uint4*>(p), f);
-  }
-};
-template <> struct WaVec<float> {
-  static constexpr int N = 4;
-  static __device__ __forceinline__ void ld(const float* p, float* f) {
-    const float4 v = *reinterpret_cast<const float4*>(p);
-    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
-  }
-};
-
-template <typename T, int REP, int NV>
-__global__ __launch_bounds__(64 * WA_NW) void window_attn_keys_kernel(WinAttnParams p) {
+template <typename T, int REP, int NV, int NW>
+__global__ __launch_bounds__(64 * NW) void window_attn_keys_kernel(WinAttnParams p) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x, g = blockIdx.y;
   if (t >= p.cu_q[p.B]) return;
   const int b = wa_seq_of_row(p.cu_q, p.B, t);
   const int D = p.D, Dv = p.Dv, rep = p.H / p.G;
-  const int r0 = blockIdx.z * REP;                 // first head of the group this block serves
+  const int sp = blockIdx.z % p.ns;                // this block's share of the key windows
+  const int r0 = (blockIdx.z / p.ns) * REP;        // first head of the group this block serves
   const int nr = min(REP, rep - r0);
   float* qs = lds;                                 // [REP][D]
-  float* ws = qs + REP * D + wave * REP * 64;      // per wave [REP][64]
-  for (int i = threadIdx.x; i < nr * D; i += blockDim.x)
-    qs[i] = Act<T>::ld((const T*)p.q + (size_t)t * p.H * D + (size_t)(g * rep + r0) * D + i);
+  float* ws = qs + REP * D + wave * (REP + 1) * 64;   // per wave: weights [REP][64] ...
+  int* rs = reinterpret_cast<int*>(ws + REP * 64);    // ... and the keys' cache rows [64]
+  for (int i = threadIdx.x; i < REP * D; i += blockDim.x)
+    qs[i] = i < nr * D ? Act<T>::ld((const T*)p.q + (size_t)t * p.H * D + (size_t)(g * rep + r0) * D + i)
+                       : 0.f;
   __syncthreads();
   const int pq = p.pos[t];
   const int hi = min(pq, p.ctx[b] - 1);
@@ -154,41 +173,69 @@ __global__ __launch_bounds__(64 * WA_NW) void window_attn_keys_kernel(WinAttnPar
   const int w_lo = lo >> 6, w_hi = hi >> 6;
   const int n1 = p.window > 0 ? min((min(p.keep_first, lo) + 63) >> 6, w_lo) : 0;
   const int nwin = hi >= 0 ? n1 + (w_hi - w_lo + 1) : 0;
-  const int* bt = p.bt + (size_t)b * p.max_blocks;
-  const T* kc = (const T*)p.kc;
-  const T* vc = (const T*)p.vc;
+  const WA_GLOBAL int* bt = (const WA_GLOBAL int*)p.bt + (size_t)b * p.max_blocks;
+  const WA_GLOBAL T* kc = (const WA_GLOBAL T*)p.kc;
+  const WA_GLOBAL T* vc = (const WA_GLOBAL T*)p.vc;
   const size_t GD = (size_t)p.G * D, GDv = (size_t)p.G * Dv;
-  float m[REP], l[REP], acc[REP][NV];
+  constexpr int VN = GAct<T>::N;
+  // value accumulators. NV > 0: a lane owns the output columns lane + 64 i.
+  // NV == 0 (Dv / VN a power of two up to 64): LPR = Dv / VN lanes cover a value
+  // row in 16-byte runs, so one load instruction brings 64 / LPR whole rows;
+  // a lane sums its run over the rows of its lane group, and the groups are
+  // added once at the end.
+  constexpr bool ROWS = NV == 0;
+  constexpr int NA = ROWS ? VN : NV;
+  const int LPR = ROWS ? Dv / VN : 64;
+  const int vrg = lane / LPR, vch = (lane % LPR) * VN;
+  float m[REP], l[REP], acc[REP][NA];
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
     m[r] = -INFINITY;
     l[r] = 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) acc[r][i] = 0.f;
+    for (int i = 0; i < NA; ++i) acc[r][i] = 0.f;
   }
-  const bool vec = D % WaVec<T>::N == 0;
-  for (int wk = wave; wk < nwin; wk += WA_NW) {
+  constexpr int KU = NW > 4 ? 4 : 8;                 // key chunks in flight per lane
+  constexpr int VU = NV > 2 ? 4 : 8;                 // value rows in flight per lane (column form)
+  const bool vec = D % VN == 0;
+  for (int wk = sp * NW + wave; wk < nwin; wk += p.ns * NW) {
     const int k0 = (wk < n1 ? wk : w_lo + (wk - n1)) << 6;
     const int j = k0 + lane;
     const bool seen = j <= hi && (p.window <= 0 || pq - j < p.window || j < p.keep_first);
+    // every lane names a valid cache row (past the end: the last key's), so the
+    // value phase below reads without bounds tests; unseen keys weigh zero
+    const int jc = min(j, hi);
+    const long row = min(max((long)bt[jc / p.blk] * p.blk + jc % p.blk, 0L), p.cache_rows - 1);
+    rs[lane] = (int)row;
     float s[REP];
 #pragma unroll
     for (int r = 0; r < REP; ++r) s[r] = 0.f;
     if (seen) {
-      const long row = min(max((long)bt[j / p.blk] * p.blk + j % p.blk, 0L), p.cache_rows - 1);
-      const T* kr = kc + (size_t)row * GD + (size_t)g * D;
+      const WA_GLOBAL T* kr = kc + (size_t)row * GD + (size_t)g * D;
       if (vec) {
-        for (int e = 0; e < D; e += WaVec<T>::N) {
-          float f[WaVec<T>::N];
-          WaVec<T>::ld(kr + e, f);
+        int e = 0;
+        for (; e + KU * VN <= D; e += KU * VN) {
+          float f[KU][VN];
+#pragma unroll
+          for (int c = 0; c < KU; ++c) GAct<T>::ldv(kr + e + c * VN, f[c]);
+#pragma unroll
+          for (int c = 0; c < KU; ++c)
+#pragma unroll
+            for (int r = 0; r < REP; ++r)
+#pragma unroll
+              for (int i = 0; i < VN; ++i) s[r] += qs[r * D + e + c * VN + i] * f[c][i];
+        }
+        for (; e < D; e += VN) {
+          float f[VN];
+          GAct<T>::ldv(kr + e, f);
 #pragma unroll
           for (int r = 0; r < REP; ++r)
 #pragma unroll
-            for (int i = 0; i < WaVec<T>::N; ++i) s[r] += qs[r * D + e + i] * f[i];
+            for (int i = 0; i < VN; ++i) s[r] += qs[r * D + e + i] * f[i];
         }
       } else {
         for (int e = 0; e < D; ++e) {
-          const float f = Act<T>::ld(kr + e);
+          const float f = GAct<T>::ld(kr + e);
 #pragma unroll
           for (int r = 0; r < REP; ++r) s[r] += qs[r * D + e] * f;
         }
@@ -211,57 +258,120 @@ __global__ __launch_bounds__(64 * WA_NW) void window_attn_keys_kernel(WinAttnPar
 #pragma unroll
     for (int r = 0; r < REP; ++r)
 #pragma unroll
-      for (int i = 0; i < NV; ++i) acc[r][i] *= alpha[r];
+      for (int i = 0; i < NA; ++i) acc[r][i] *= alpha[r];
     const int nk = min(64, hi - k0 + 1);
-    for (int kk = 0; kk < nk; ++kk) {
-      const int jj = k0 + kk;
-      const long row = min(max((long)bt[jj / p.blk] * p.blk + jj % p.blk, 0L), p.cache_rows - 1);
-      const T* vr = vc + (size_t)row * GDv + (size_t)g * Dv;
-      float v[NV];
+    if constexpr (ROWS) {
+      const int rpi = 64 / LPR;                        // rows per load instruction
+      for (int i0 = 0; i0 * rpi < nk; i0 += 4) {       // rows past nk weigh zero
+        float v[4][VN];
+        int key[4];
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int e = lane + 64 * i;
-        v[i] = e < Dv ? Act<T>::ld(vr + e) : 0.f;
+        for (int c = 0; c < 4; ++c) {
+          key[c] = min((i0 + c) * rpi + vrg, 63);
+          GAct<T>::ldv(vc + (size_t)rs[key[c]] * GDv + (size_t)g * Dv + vch, v[c]);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          if ((i0 + c) * rpi >= 64) break;             // uniform: fewer than four loads left
+#pragma unroll
+          for (int r = 0; r < REP; ++r) {
+            const float w = ws[r * 64 + key[c]];
+#pragma unroll
+            for (int i = 0; i < VN; ++i) acc[r][i] += w * v[c][i];
+          }
+        }
+      }
+    } else
+    for (int kk = 0; kk < nk; kk += VU) {              // rows past nk weigh zero
+      float v[VU][NA];
+#pragma unroll
+      for (int c = 0; c < VU; ++c) {
+        const WA_GLOBAL T* vr = vc + (size_t)rs[kk + c] * GDv + (size_t)g * Dv;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+          const int e = lane + 64 * i;
+          v[c][i] = e < Dv ? GAct<T>::ld(vr + e) : 0.f;
+        }
       }
 #pragma unroll
-      for (int r = 0; r < REP; ++r) {
-        const float w = ws[r * 64 + kk];
+      for (int c = 0; c < VU; ++c)
 #pragma unroll
-        for (int i = 0; i < NV; ++i) acc[r][i] += w * v[i];
-      }
+        for (int r = 0; r < REP; ++r) {
+          const float w = ws[r * 64 + kk + c];
+#pragma unroll
+          for (int i = 0; i < NA; ++i) acc[r][i] += w * v[c][i];
+        }
     }
     __builtin_amdgcn_wave_barrier();
   }
+  if constexpr (ROWS) {
+    // add the lane groups: afterwards lanes 0 .. LPR - 1 hold the wave's sums
+    for (int o = LPR; o < 64; o <<= 1)
+#pragma unroll
+      for (int r = 0; r < REP; ++r)
+#pragma unroll
+        for (int i = 0; i < NA; ++i) acc[r][i] += __shfl_xor(acc[r][i], o, 64);
+  }
   // merge the waves' partials in wave order
   __syncthreads();                                   // qs / ws are free
-  float* mm = lds;                                   // [WA_NW][REP]
-  float* ll = mm + WA_NW * REP;                      // [WA_NW][REP]
-  float* aa = ll + WA_NW * REP;                      // [WA_NW][REP][NV * 64]
+  float* mm = lds;                                   // [NW][REP]
+  float* ll = mm + NW * REP;                         // [NW][REP]
+  float* aa = ll + NW * REP;                         // [NW][REP][Dv]
   if (lane == 0)
 #pragma unroll
     for (int r = 0; r < REP; ++r) { mm[wave * REP + r] = m[r]; ll[wave * REP + r] = l[r]; }
 #pragma unroll
   for (int r = 0; r < REP; ++r)
 #pragma unroll
-    for (int i = 0; i < NV; ++i) aa[((wave * REP + r) * NV + i) * 64 + lane] = acc[r][i];
+    for (int i = 0; i < NA; ++i) {
+      const int e = ROWS ? vch + i : lane + 64 * i;
+      if (e < Dv && (!ROWS || lane < LPR)) aa[(size_t)(wave * REP + r) * Dv + e] = acc[r][i];
+    }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < nr * NV * 64; idx += blockDim.x) {
-    const int r = idx / (NV * 64), c = idx % (NV * 64), i = c >> 6, ln = c & 63;
-    const int e = ln + 64 * i;
-    if (e >= Dv) continue;
+  for (int idx = threadIdx.x; idx < nr * Dv; idx += blockDim.x) {
+    const int r = idx / Dv, e = idx - r * Dv;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < WA_NW; ++w) M = fmaxf(M, mm[w * REP + r]);
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, mm[w * REP + r]);
     float num = 0.f, den = 0.f;
 #pragma unroll
-    for (int w = 0; w < WA_NW; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float mw = mm[w * REP + r];
       const float f = mw == -INFINITY ? 0.f : expf(mw - M);
-      num += f * aa[((w * REP + r) * NV + i) * 64 + ln];
+      num += f * aa[(size_t)(w * REP + r) * Dv + e];
       den += f * ll[w * REP + r];
     }
-    float out = den > 0.f ? num / den : 0.f;
     const int h = g * rep + r0 + r;
+    if (p.ns > 1) {                                  // the combine launch finishes the row
+      float* pr = p.part + (((size_t)t * p.H + h) * p.ns + sp) * (Dv + 2);
+      if (e == 0) { pr[0] = M; pr[1] = den; }
+      pr[2 + e] = num;
+      continue;
+    }
+    float out = den > 0.f ? num / den : 0.f;
+    if (p.gate)
+      out *= sigmoid_f(Act<T>::ld((const T*)p.gate + (size_t)t * p.gate_ld + (size_t)h * Dv + e));
+    Act<T>::st((T*)p.o + (size_t)t * p.H * Dv + (size_t)h * Dv + e, out);
+  }
+}
+
+// Merge of the key splits of a row: partials (max, sum, accumulator[Dv]) in
+// split order, then the output gate.
+template <typename T>
+__global__ __launch_bounds__(128) void window_attn_combine_kernel(WinAttnParams p) {
+  const int t = blockIdx.x, h = blockIdx.y, Dv = p.Dv;
+  const float* pr = p.part + ((size_t)t * p.H + h) * p.ns * (Dv + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < p.ns; ++s) M = fmaxf(M, pr[(size_t)s * (Dv + 2)]);
+  for (int e = threadIdx.x; e < Dv; e += blockDim.x) {
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < p.ns; ++s) {
+      const float* ps = pr + (size_t)s * (Dv + 2);
+      const float f = ps[0] == -INFINITY ? 0.f : expf(ps[0] - M);
+      num += f * ps[2 + e];
+      den += f * ps[1];
+    }
+    float out = den > 0.f ? num / den : 0.f;
     if (p.gate)
       out *= sigmoid_f(Act<T>::ld((const T*)p.gate + (size_t)t * p.gate_ld + (size_t)h * Dv + e));
     Act<T>::st((T*)p.o + (size_t)t * p.H * Dv + (size_t)h * Dv + e, out);
@@ -269,9 +379,8 @@ __global__ __launch_bounds__(64 * WA_NW) void window_attn_keys_kernel(WinAttnPar
 }
 
 // ------------------------------------------------------------ prompt portions
-#define WM_THREADS 256
-#define WM_WAVES 4
 #define WM_TILE 64
+#define WM_MAXPG 2048                // block-table entries of a sequence kept in LDS
 
 typedef short wm_v4s __attribute__((ext_vector_type(4)));
 
@@ -287,9 +396,11 @@ __device__ __forceinline__ float tanh_fast(float z) {
   return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.885390081777927f * z));
 }
 
-template <int DK, int DV>
-__global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnParams p) {
+template <int DK, int DV, int WM_WAVES>
+__global__ __launch_bounds__(64 * WM_WAVES) void window_attn_mfma_kernel(WinAttnParams p) {
   __shared__ __attribute__((aligned(16))) WinMfmaSmem<DK, DV> sm;
+  __shared__ int pages[WM_MAXPG];
+  constexpr int WM_THREADS = 64 * WM_WAVES;
   constexpr int NS = DK / 16, NDT = DV / 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5;
   const int head = blockIdx.y, b = blockIdx.z;
@@ -334,31 +445,42 @@ __global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnPar
   float m_run = -1e30f, l_run = 0.f;
   constexpr int CHK = DK / 8, CHV = DV / 8;
   const size_t kst = (size_t)p.G * DK, vst = (size_t)p.G * DV;
-  const bf16_t* kbase = (const bf16_t*)p.kc + (size_t)g * DK;
-  const bf16_t* vbase = (const bf16_t*)p.vc + (size_t)g * DV;
-  const int* bt = p.bt + (size_t)b * p.max_blocks;
+  const WA_GLOBAL bf16_t* kbase = (const WA_GLOBAL bf16_t*)p.kc + (size_t)g * DK;
+  const WA_GLOBAL bf16_t* vbase = (const WA_GLOBAL bf16_t*)p.vc + (size_t)g * DV;
+  const WA_GLOBAL int* bt = (const WA_GLOBAL int*)p.bt + (size_t)b * p.max_blocks;
+  // the pages of this workgroup's key range, looked up once
+  const int npg = (kend + p.blk - 1) / p.blk;
+  const bool pg_lds = npg <= WM_MAXPG;
+  if (pg_lds) {
+    for (int i = threadIdx.x; i < npg; i += WM_THREADS) pages[i] = bt[i];
+    __syncthreads();
+  }
   const float scale_log2 = p.scale * 1.4426950408889634f;
   const float cap_log2 = p.cap * 1.4426950408889634f, inv_cap = p.cap > 0.f ? p.scale / p.cap : 0.f;
 
   // K / V tiles go through registers: the next tile's 16-byte chunks are
   // requested before this tile's math and stored to LDS after it
   constexpr int NKC = WM_TILE * CHK / WM_THREADS, NVC = WM_TILE * CHV / WM_THREADS;
-  uint4 pk[NKC], pv[NVC];
+  wa_u32x4 pk[NKC], pv[NVC];
   auto page_row = [&](int j) -> size_t {
-    return (size_t)min(max((long)bt[j / p.blk] * p.blk + j % p.blk, 0L), p.cache_rows - 1);
+    const int pi = j / p.blk;
+    const long pg = pg_lds ? pages[pi] : bt[pi];
+    return (size_t)min(max(pg * p.blk + (j - pi * p.blk), 0L), p.cache_rows - 1);
   };
   auto fetch = [&](int kt) {
 #pragma unroll
     for (int j = 0; j < NKC; ++j) {
       const int c = threadIdx.x + WM_THREADS * j, kr = c / CHK, cc = (c - kr * CHK) * 8;
-      pk[j] = kt + kr < kend ? *reinterpret_cast<const uint4*>(kbase + page_row(kt + kr) * kst + cc)
-                             : make_uint4(0, 0, 0, 0);
+      pk[j] = kt + kr < kend
+                  ? *reinterpret_cast<const WA_GLOBAL wa_u32x4*>(kbase + page_row(kt + kr) * kst + cc)
+                  : wa_u32x4{0, 0, 0, 0};
     }
 #pragma unroll
     for (int j = 0; j < NVC; ++j) {
       const int c = threadIdx.x + WM_THREADS * j, kr = c / CHV, cc = (c - kr * CHV) * 8;
-      pv[j] = kt + kr < kend ? *reinterpret_cast<const uint4*>(vbase + page_row(kt + kr) * vst + cc)
-                             : make_uint4(0, 0, 0, 0);
+      pv[j] = kt + kr < kend
+                  ? *reinterpret_cast<const WA_GLOBAL wa_u32x4*>(vbase + page_row(kt + kr) * vst + cc)
+                  : wa_u32x4{0, 0, 0, 0};
     }
   };
   auto tile_at = [&](int i) { return i < n1 ? i * WM_TILE : lo_t + (i - n1) * WM_TILE; };
@@ -369,12 +491,12 @@ __global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnPar
 #pragma unroll
     for (int j = 0; j < NKC; ++j) {
       const int c = threadIdx.x + WM_THREADS * j, kr = c / CHK, cc = (c - kr * CHK) * 8;
-      *reinterpret_cast<uint4*>(&sm.k[kr][cc]) = pk[j];
+      *reinterpret_cast<wa_u32x4*>(&sm.k[kr][cc]) = pk[j];
     }
 #pragma unroll
     for (int j = 0; j < NVC; ++j) {
       const int c = threadIdx.x + WM_THREADS * j, kr = c / CHV, cc = (c - kr * CHV) * 8;
-      *reinterpret_cast<uint4*>(&sm.v[kr][cc]) = pv[j];
+      *reinterpret_cast<wa_u32x4*>(&sm.v[kr][cc]) = pv[j];
     }
     __syncthreads();
     if (ti + 1 < ntiles) fetch(tile_at(ti + 1));
@@ -398,21 +520,38 @@ __global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnPar
     bf16x8 pf[2][2];
     {
       float mx = -INFINITY;
+      // a tile that every row of this wave sees whole needs no per-score tests
+      const bool whole = kt + WM_TILE - 1 <= wpos_lo && kt + WM_TILE <= kend &&
+                         (p.window <= 0 || wpos_hi - kt < p.window || kt + WM_TILE <= p.keep_first);
+      if (whole) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int key = kt + 32 * t + (j & 3) + 8 * (j >> 2) + 4 * h;
-          float sv = p.cap > 0.f ? cap_log2 * tanh_fast(st[t][j] * inv_cap) : st[t][j] * scale_log2;
-          if (key >= kend || key > qpos ||
-              (p.window > 0 && qpos - key >= p.window && key >= p.keep_first))
-            sv = -INFINITY;
-          st[t][j] = sv;
-          mx = fmaxf(mx, sv);
-        }
+          for (int j = 0; j < 16; ++j) {
+            const float sv = p.cap > 0.f ? cap_log2 * tanh_fast(st[t][j] * inv_cap)
+                                         : st[t][j] * scale_log2;
+            st[t][j] = sv;
+            mx = fmaxf(mx, sv);
+          }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const int key = kt + 32 * t + (j & 3) + 8 * (j >> 2) + 4 * h;
+            float sv = p.cap > 0.f ? cap_log2 * tanh_fast(st[t][j] * inv_cap) : st[t][j] * scale_log2;
+            if (key >= kend || key > qpos ||
+                (p.window > 0 && qpos - key >= p.window && key >= p.keep_first))
+              sv = -INFINITY;
+            st[t][j] = sv;
+            mx = fmaxf(mx, sv);
+          }
+      }
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = exp2f(m_run - m_new);
+      // the hardware's exp2: the arguments are <= 0, and what falls below the
+      // normal range may flush to zero
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       float ls = 0.f;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -420,7 +559,7 @@ __global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnPar
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            const float e = exp2f(st[t][8 * s2 + j] - m_new);
+            const float e = __builtin_amdgcn_exp2f(st[t][8 * s2 + j] - m_new);
             ls += e;
             pf[t][s2][j] = (__bf16)e;
           }
@@ -482,10 +621,16 @@ __global__ __launch_bounds__(WM_THREADS) void window_attn_mfma_kernel(WinAttnPar
 
 int window_attention_mfma(const WinAttnParams& p, int max_q, hipStream_t st) {
   if (max_q <= 0) return 0;
-  const dim3 grid((max_q + WM_WAVES * 32 - 1) / (WM_WAVES * 32), p.H, p.B);
+  // 128-row blocks when they alone fill the GPU several times over, else 64-row blocks
+  const long wg4 = (long)((max_q + 127) / 128) * p.H * p.B;
+  const int waves = wg4 >= 1024 ? 4 : 2;
+  const dim3 grid((max_q + waves * 32 - 1) / (waves * 32), p.H, p.B);
 #define GO(A, C)                                                                              \
   if (p.D == A && p.Dv == C) {                                                                \
-    hipLaunchKernelGGL((window_attn_mfma_kernel<A, C>), grid, dim3(WM_THREADS), 0, st, p);    \
+    if (waves == 4)                                                                           \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<A, C, 4>), grid, dim3(256), 0, st, p);      \
+    else                                                                                      \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<A, C, 2>), grid, dim3(128), 0, st, p);      \
     return (int)hipGetLastError();                                                            \
   }
   GO(64, 64) GO(128, 64) GO(64, 128) GO(128, 128)
@@ -518,7 +663,7 @@ extern "C" int loqa_window_attention(const void* q, int dt, const void* kc, cons
                                      int max_blocks, const void* pos, const void* gate, long gate_ld,
                                      float scale, float cap, int window, int keep_first, int B,
                                      int T, int H, int G, int D, int Dv, int max_q, int mfma,
-                                     void* o, hipStream_t st) {
+                                     void* o, int ns, void* part, hipStream_t st) {
   if (T <= 0) return 0;
   if (B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > 512 || Dv <= 0 || Dv > 512 || blk <= 0)
     return (int)hipErrorInvalidValue;
@@ -528,29 +673,52 @@ extern "C" int loqa_window_attention(const void* q, int dt, const void* kc, cons
   p.max_blocks = max_blocks; p.pos = (const int*)pos; p.gate = gate; p.gate_ld = gate_ld;
   p.scale = scale; p.cap = cap; p.window = window; p.keep_first = keep_first;
   p.B = B; p.T = T; p.H = H; p.G = G; p.D = D; p.Dv = Dv; p.o = o;
+  p.ns = 1; p.part = nullptr;
   // the matrix-core form reads the gate in 8-byte runs
   const bool gate_ok = !gate || (gate_ld % 4 == 0 && ((size_t)gate & 7) == 0);
   if (mfma && dt == 0 && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) && gate_ok)
     return window_attention_mfma(p, max_q, st);
   const int rep = H / G;
-  const int nv = Dv <= 128 ? 2 : 8;
+  // value layout: whole rows in 16-byte runs when Dv / (elements per run) is a
+  // power of two up to 64, else a column per lane (2 or 8 columns)
+  const int vn = dt == 0 ? 8 : 4, lpr = Dv / vn;
+  const bool rows = Dv % vn == 0 && lpr <= 64 && (lpr & (lpr - 1)) == 0;
+  const int nv = rows ? 0 : (Dv <= 128 ? 2 : 8);
   int R = rep >= 8 ? 8 : (rep >= 4 ? 4 : (rep >= 2 ? 2 : 1));
   if (nv == 8 && R > 4) R = 4;
-  const dim3 grid(T, G, (rep + R - 1) / R);
-  const size_t lds1 = (size_t)(R * D + WA_NW * R * 64) * 4;
-  const size_t lds2 = (size_t)(2 * WA_NW * R + WA_NW * R * nv * 64) * 4;
-  const size_t lds = lds1 > lds2 ? lds1 : lds2;
+  if (ns > 1 && part) { p.ns = ns; p.part = (float*)part; }
+  const dim3 grid(T, G, (rep + R - 1) / R * p.ns);
+  // few workgroups (decode steps): 16 waves share a row's keys, else 4
+  auto lds_of = [&](int nw) {
+    const size_t a = (size_t)(R * D + nw * (R + 1) * 64) * 4;
+    const size_t b = (size_t)(2 * nw * R + nw * R * Dv) * 4;
+    return a > b ? a : b;
+  };
+  int nw = rows && p.ns == 1 && (long)grid.x * grid.y * grid.z < 256 ? 16 : 4;
+  if (lds_of(nw) > 64 * 1024) nw = 4;
+  const size_t lds = lds_of(nw);
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
-#define GO(TT, RR, NN)                                                                         \
-  hipLaunchKernelGGL((window_attn_keys_kernel<TT, RR, NN>), grid, dim3(64 * WA_NW), lds, st, p)
-#define BY_R(TT, NN)                                                                           \
+#define GO(TT, RR, NN, WW)                                                                     \
+  hipLaunchKernelGGL((window_attn_keys_kernel<TT, RR, NN, WW>), grid, dim3(64 * WW), lds, st, p)
+#define BY_R(TT, NN, WW)                                                                       \
   do {                                                                                         \
-    if (R == 8) GO(TT, 8, NN); else if (R == 4) GO(TT, 4, NN);                                 \
-    else if (R == 2) GO(TT, 2, NN); else GO(TT, 1, NN);                                        \
+    if (R == 8) GO(TT, 8, NN, WW); else if (R == 4) GO(TT, 4, NN, WW);                         \
+    else if (R == 2) GO(TT, 2, NN, WW); else GO(TT, 1, NN, WW);                                \
   } while (0)
-  if (dt == 0) { if (nv == 2) BY_R(bf16_t, 2); else BY_R(bf16_t, 8); }
-  else { if (nv == 2) BY_R(float, 2); else BY_R(float, 8); }
+#define BY_V(TT)                                                                               \
+  do {                                                                                         \
+    if (nv == 0 && nw == 16) BY_R(TT, 0, 16); else if (nv == 0) BY_R(TT, 0, 4);                \
+    else if (nv == 2) BY_R(TT, 2, 4); else BY_R(TT, 8, 4);                                     \
+  } while (0)
+  if (dt == 0) BY_V(bf16_t); else BY_V(float);
+#undef BY_V
 #undef BY_R
 #undef GO
+  if (p.ns > 1) {
+    if (dt == 0)
+      hipLaunchKernelGGL(window_attn_combine_kernel<bf16_t>, dim3(T, H), dim3(128), 0, st, p);
+    else
+      hipLaunchKernelGGL(window_attn_combine_kernel<float>, dim3(T, H), dim3(128), 0, st, p);
+  }
   return (int)hipGetLastError();
 }

@@ -334,7 +334,7 @@ class MovinexModel:
         gate = u[:, L["g_off"]:L["g_off"] + H * Dv] if m.gate else None
         o = seqmix.window_attention(q, kc, vc, meta.cu_q, meta.ctx_lens, meta.block_tables,
                                     meta.positions, m.scale, m.softcap, m.window, m.keep_first,
-                                    gate, H, G, D, Dv, meta.max_q)
+                                    gate, H, G, D, Dv, meta.max_q, max_ctx=meta.max_ctx)
         return ops.linear(o, L["wo"])
 
     def _mamba2(self, r, m, L, h, meta, cache) -> torch.Tensor:

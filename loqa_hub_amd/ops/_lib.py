@@ -239,7 +239,7 @@ _SEQMIX_SIGS = {
     "loqa_qk_prep_append": [_vp, _i, _l, _i, _i, _i, _i, _i, _vp, _i, _i, _f, _f, _i, _vp, _vp,
                             _vp, _i, _i, _vp, _vp, _i, _vp],
     "loqa_window_attention": [_vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _l, _f, _f,
-                              _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp],
+                              _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp],
     "loqa_mamba2_prep": [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp,
                          _vp, _i, _i, _vp, _vp, _vp],
 }

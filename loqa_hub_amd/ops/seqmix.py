@@ -698,7 +698,8 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      cu_q: torch.Tensor, ctx_lens: torch.Tensor, block_tables: torch.Tensor,
                      positions: torch.Tensor, scale: float, softcap: float, window: int,
                      keep_first: int, gate: torch.Tensor | None, H: int, G: int, D: int, Dv: int,
-                     max_q: int = 0, matrix_cores: bool | None = None) -> torch.Tensor:
+                     max_q: int = 0, matrix_cores: bool | None = None, max_ctx: int = 0,
+                     key_splits: int | None = None) -> torch.Tensor:
     """Softmax attention over paged K [blocks, BLK, G D] and V [blocks, BLK,
     G Dv] (query head h reads key/value head h // (H / G)): score = q . k *
     scale, soft-capped to cap tanh(score / cap) when ``softcap`` > 0; a query at
@@ -707,7 +708,10 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     be a column slice) multiplies the output by sigmoid(gate) per entry. q
     [T, H D] -> [T, H Dv]. Rows find their sequence through ``cu_q`` and their
     keys through the block table, so prompt portions, decode tokens and mixed
-    batches are one launch. Scores, softmax and accumulators are f32."""
+    batches are one launch. Scores, softmax and accumulators are f32. A step
+    with few rows over long contexts (``max_ctx``) deals each row's keys out to
+    ``key_splits`` workgroups (chosen here when None) and merges their partial
+    results in a second launch."""
     if not q.is_cuda:
         return ref.window_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions,
                                     scale, softcap, window, keep_first, gate, H, G, D, Dv, q.dtype)
@@ -730,12 +734,24 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         matrix_cores = max_q >= 16
     mfma = bool(matrix_cores) and q.dtype == torch.bfloat16 and D in WINDOW_MFMA_D \
         and Dv in WINDOW_MFMA_D
+    part = None
+    if key_splits is None:
+        # 64-key windows a row can have, four (one per wave) to a workgroup
+        keys = max(int(max_ctx), 1) if window <= 0 else min(max(int(max_ctx), 1),
+                                                           window + 64 + keep_first)
+        key_splits = 1 if mfma or T * G >= 256 else \
+            max(1, min(16, -(-keys // 256), 512 // max(1, T * G)))
+    if key_splits > 1 and not mfma:
+        part = torch.empty(T * H * key_splits * (Dv + 2), dtype=torch.float32, device=q.device)
+    else:
+        key_splits = 1
     if T:
         check(kernels().loqa_window_attention(
             ptr(q), _dt(q), ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0],
             ptr(cu_q), ptr(ctx_lens), ptr(block_tables), block_tables.shape[1], ptr(positions),
             ptr(gate), gs, float(scale), float(softcap), int(window), int(keep_first), B, T, H, G,
-            D, Dv, int(max_q), int(mfma), ptr(o), stream_ptr(q)), "window_attention")
+            D, Dv, int(max_q), int(mfma), ptr(o), int(key_splits), ptr(part), stream_ptr(q)),
+            "window_attention")
     return o
 
 

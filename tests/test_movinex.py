@@ -190,7 +190,7 @@ def _paged(k, v, lens, blk, device, seed=0):
 
 
 def _attention_case(device, dtype, H, G, D, Dv, window, keep, cap, lens, feeds, gate, mfma=None,
-                    spike=None, seed=2, gate_pad=(2, 5)):
+                    spike=None, seed=2, gate_pad=(2, 5), splits=None):
     """Sequences of ``lens`` keys whose last ``feeds`` positions are this step's
     queries; compares seqmix.window_attention with the oracle. ``spike`` =
     (distance back, strength): the key that far behind each query's position
@@ -223,7 +223,7 @@ def _attention_case(device, dtype, H, G, D, Dv, window, keep, cap, lens, feeds, 
     got = seqmix.window_attention(
         q.to(device, dtype), kc.to(dtype), vc.to(dtype), cu, ctx, bt, pos, scale, cap, window, keep,
         gt.to(device)[:, g0:g0 + H * Dv] if gate else None, H, G, D, Dv, max(feeds),
-        matrix_cores=mfma)
+        matrix_cores=mfma, max_ctx=max(lens), key_splits=splits)
     want = []
     for b, n in enumerate(lens):
         o = O.softmax_attention(qs[b].double().view(n, H, D), ks[b].double().view(n, G, D),
@@ -646,6 +646,24 @@ def test_window_attention_matrix_cores(H, G, D, Dv, window, keep, cap):
         scale = float(want.abs().max())
         assert (a - want).abs().max() < 0.03 * scale and (b - want).abs().max() < 0.03 * scale
         assert (a - b).abs().max() < 0.03 * scale
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("splits", [None, 2, 5, 16])
+def test_window_attention_key_splits(dtype, splits):
+    """Decode rows whose keys are dealt out to several workgroups and merged by
+    the combine launch: long and short contexts side by side, a window with
+    kept first tokens, an output gate, a far key that must be found."""
+    tol = 2e-5 if dtype == torch.float32 else 0.03
+    for window, keep, cap in ((0, 0, 0.0), (200, 70, 20.0)):
+        got, want = _attention_case("cuda", dtype, 8, 2, 64, 64, window, keep, cap,
+                                    [1500, 3, 700, 64, 65], [1, 1, 1, 1, 2], True, mfma=False,
+                                    gate_pad=(8, 16), splits=splits)
+        assert (got - want).abs().max() < tol * max(1.0, float(want.abs().max()))
+    got, want = _attention_case("cuda", torch.float32, 2, 1, 16, 16, 0, 0, 0.0, [1500], [1], False,
+                                mfma=False, spike=(1234, 40.0), splits=splits)
+    assert (got - want).abs().max() < 2e-5
 
 
 @pytest.mark.gpu
