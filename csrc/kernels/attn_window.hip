@@ -78,9 +78,32 @@ template <> struct GAct<float> {
   }
 };
 
+// Sum over groups of `gs` neighbouring lanes (a power of two): data-parallel
+// moves inside rows of 16 lanes, shuffles above; every lane gets its group's sum.
+template <int CTRL> __device__ __forceinline__ float wa_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float wa_group_sum(float v, int gs) {
+  if (gs >= 2) v += wa_dpp<0xB1>(v);              // lanes 1 0 3 2 of each four
+  if (gs >= 4) v += wa_dpp<0x4E>(v);              // lanes 2 3 0 1 of each four
+  if (gs >= 8) v += wa_dpp<0x141>(v);             // the other four of each eight (mirror)
+  if (gs >= 16) v += wa_dpp<0x140>(v);            // the other eight of each sixteen (mirror)
+  if (gs >= 32) v += __shfl_xor(v, 16, 64);
+  if (gs >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// The sequence of flat row t: the number of feed starts cu_q[1 .. B - 1] at or
+// before t. Every lane tests one start, so a batch of up to 64 sequences costs
+// one round trip instead of a chain of dependent loads (all lanes must be active).
 __device__ __forceinline__ int wa_seq_of_row(const int* __restrict__ cu_q, int B, int t) {
+  const int lane = threadIdx.x & 63;
   int b = 0;
-  while (b + 1 < B && t >= cu_q[b + 1]) ++b;
+  for (int base = 1; base < B; base += 64) {
+    const int i = base + lane;
+    const bool at_or_before = i < B && cu_q[i] <= t;
+    b += __popcll(__ballot(at_or_before));
+  }
   return b;
 }
 
@@ -195,50 +218,64 @@ __global__ __launch_bounds__(64 * NW) void window_attn_keys_kernel(WinAttnParams
 #pragma unroll
     for (int i = 0; i < NA; ++i) acc[r][i] = 0.f;
   }
-  constexpr int KU = NW > 4 ? 4 : 8;                 // key chunks in flight per lane
+  constexpr int KU = NW > 4 ? 4 : 8;                 // key / value row loads in flight per lane
+  // key layout: LPK = D / VN lanes cover a key row in 16-byte runs when that is
+  // a power of two up to 64 (else a lane per key, element by element); lane
+  // group krg reads the rows krg, krg + 64 / LPK, ..., and the lane whose place
+  // in the group equals the load's number owns that key from then on
+  const int LPKc = D / VN;
+  const bool krows = D % VN == 0 && LPKc <= 64 && (LPKc & (LPKc - 1)) == 0;
+  const int LPK = krows ? LPKc : 64;
+  const int krg = lane / LPK, kit = lane % LPK, kch = kit * VN;
+  const int jl = krows ? kit * (64 / LPK) + krg : lane;   // the window's key this lane owns
+  float qreg[REP][VN];
+#pragma unroll
+  for (int r = 0; r < REP; ++r)
+#pragma unroll
+    for (int i = 0; i < VN; ++i) qreg[r][i] = krows ? qs[r * D + kch + i] : 0.f;
   constexpr int VU = NV > 2 ? 4 : 8;                 // value rows in flight per lane (column form)
-  const bool vec = D % VN == 0;
   for (int wk = sp * NW + wave; wk < nwin; wk += p.ns * NW) {
     const int k0 = (wk < n1 ? wk : w_lo + (wk - n1)) << 6;
-    const int j = k0 + lane;
+    const int j = k0 + jl;
     const bool seen = j <= hi && (p.window <= 0 || pq - j < p.window || j < p.keep_first);
     // every lane names a valid cache row (past the end: the last key's), so the
-    // value phase below reads without bounds tests; unseen keys weigh zero
+    // loads below need no bounds tests; unseen keys weigh zero
     const int jc = min(j, hi);
     const long row = min(max((long)bt[jc / p.blk] * p.blk + jc % p.blk, 0L), p.cache_rows - 1);
-    rs[lane] = (int)row;
+    rs[jl] = (int)row;
     float s[REP];
 #pragma unroll
     for (int r = 0; r < REP; ++r) s[r] = 0.f;
-    if (seen) {
+    if (krows) {
+      // one load instruction brings 64 / LPK whole key rows; a lane multiplies its
+      // 16-byte run with its part of q, the group adds up, the key's owner keeps it
+      __builtin_amdgcn_wave_barrier();
+      const int rpk = 64 / LPK;
+      for (int i0 = 0; i0 < LPK; i0 += KU) {
+        float f[KU][VN];
+#pragma unroll
+        for (int c = 0; c < KU; ++c) {
+          const int kl = min((i0 + c) * rpk + krg, 63);
+          GAct<T>::ldv(kc + (size_t)rs[kl] * GD + (size_t)g * D + kch, f[c]);
+        }
+#pragma unroll
+        for (int c = 0; c < KU; ++c) {
+#pragma unroll
+          for (int r = 0; r < REP; ++r) {
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < VN; ++i) d += qreg[r][i] * f[c][i];
+            d = wa_group_sum(d, LPK);
+            if (i0 + c == kit) s[r] = d;
+          }
+        }
+      }
+    } else if (seen) {
       const WA_GLOBAL T* kr = kc + (size_t)row * GD + (size_t)g * D;
-      if (vec) {
-        int e = 0;
-        for (; e + KU * VN <= D; e += KU * VN) {
-          float f[KU][VN];
+      for (int e = 0; e < D; ++e) {
+        const float f = GAct<T>::ld(kr + e);
 #pragma unroll
-          for (int c = 0; c < KU; ++c) GAct<T>::ldv(kr + e + c * VN, f[c]);
-#pragma unroll
-          for (int c = 0; c < KU; ++c)
-#pragma unroll
-            for (int r = 0; r < REP; ++r)
-#pragma unroll
-              for (int i = 0; i < VN; ++i) s[r] += qs[r * D + e + c * VN + i] * f[c][i];
-        }
-        for (; e < D; e += VN) {
-          float f[VN];
-          GAct<T>::ldv(kr + e, f);
-#pragma unroll
-          for (int r = 0; r < REP; ++r)
-#pragma unroll
-            for (int i = 0; i < VN; ++i) s[r] += qs[r * D + e + i] * f[i];
-        }
-      } else {
-        for (int e = 0; e < D; ++e) {
-          const float f = GAct<T>::ld(kr + e);
-#pragma unroll
-          for (int r = 0; r < REP; ++r) s[r] += qs[r * D + e] * f;
-        }
+        for (int r = 0; r < REP; ++r) s[r] += qs[r * D + e] * f;
       }
     }
     float alpha[REP];
@@ -252,7 +289,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_keys_kernel(WinAttnParams
       alpha[r] = expf(m[r] - mn);
       l[r] = l[r] * alpha[r] + wave_sum(e);
       m[r] = mn;
-      ws[r * 64 + lane] = e;
+      ws[r * 64 + jl] = e;
     }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -262,17 +299,17 @@ __global__ __launch_bounds__(64 * NW) void window_attn_keys_kernel(WinAttnParams
     const int nk = min(64, hi - k0 + 1);
     if constexpr (ROWS) {
       const int rpi = 64 / LPR;                        // rows per load instruction
-      for (int i0 = 0; i0 * rpi < nk; i0 += 4) {       // rows past nk weigh zero
-        float v[4][VN];
-        int key[4];
+      for (int i0 = 0; i0 * rpi < nk; i0 += KU) {      // rows past nk weigh zero
+        float v[KU][VN];
+        int key[KU];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < KU; ++c) {
           key[c] = min((i0 + c) * rpi + vrg, 63);
           GAct<T>::ldv(vc + (size_t)rs[key[c]] * GDv + (size_t)g * Dv + vch, v[c]);
         }
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          if ((i0 + c) * rpi >= 64) break;             // uniform: fewer than four loads left
+        for (int c = 0; c < KU; ++c) {
+          if ((i0 + c) * rpi >= 64) break;             // uniform: no rows left
 #pragma unroll
           for (int r = 0; r < REP; ++r) {
             const float w = ws[r * 64 + key[c]];
@@ -462,8 +499,10 @@ __global__ __launch_bounds__(64 * WM_WAVES) void window_attn_mfma_kernel(WinAttn
   // requested before this tile's math and stored to LDS after it
   constexpr int NKC = WM_TILE * CHK / WM_THREADS, NVC = WM_TILE * CHV / WM_THREADS;
   wa_u32x4 pk[NKC], pv[NVC];
+  // page size a power of two (the usual case): shifts instead of divisions
+  const int pg_sh = (p.blk & (p.blk - 1)) == 0 ? __ffs(p.blk) - 1 : -1;
   auto page_row = [&](int j) -> size_t {
-    const int pi = j / p.blk;
+    const int pi = pg_sh >= 0 ? j >> pg_sh : j / p.blk;
     const long pg = pg_lds ? pages[pi] : bt[pi];
     return (size_t)min(max(pg * p.blk + (j - pi * p.blk), 0L), p.cache_rows - 1);
   };
@@ -694,7 +733,7 @@ extern "C" int loqa_window_attention(const void* q, int dt, const void* kc, cons
     const size_t b = (size_t)(2 * nw * R + nw * R * Dv) * 4;
     return a > b ? a : b;
   };
-  int nw = rows && p.ns == 1 && (long)grid.x * grid.y * grid.z < 256 ? 16 : 4;
+  int nw = rows && R <= 2 && p.ns == 1 && (long)grid.x * grid.y * grid.z < 256 ? 16 : 4;
   if (lds_of(nw) > 64 * 1024) nw = 4;
   const size_t lds = lds_of(nw);
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;

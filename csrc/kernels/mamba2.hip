@@ -21,9 +21,16 @@
 // neighbouring channels of a bf16 projection (16-byte loads).
 #include "seqmix.h"
 
+// The sequence of flat row t: the number of feed starts cu_q[1 .. B - 1] at or
+// before t, a lane per start (all lanes must be active).
 __device__ __forceinline__ int m2_seq_of_row(const int* __restrict__ cu_q, int B, int t) {
+  const int lane = threadIdx.x & 63;
   int b = 0;
-  while (b + 1 < B && t >= cu_q[b + 1]) ++b;
+  for (int base = 1; base < B; base += 64) {
+    const int i = base + lane;
+    const bool at_or_before = i < B && cu_q[i] <= t;
+    b += __popcll(__ballot(at_or_before));
+  }
   return b;
 }
 
