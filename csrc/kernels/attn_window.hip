@@ -33,8 +33,8 @@
 // workgroups per row, whose partial triples a small combine launch merges.
 //
 // window_attn_mfma_kernel (bf16, D and Dv in {64, 128}; prompt portions): a
-// workgroup per (64 or 128 query rows of one sequence, query head); each wave
-// owns 32 rows. The block-table entries of the key range go to LDS once. K and V tiles of 64 keys are gathered from the pages into LDS for all
+// workgroup per (64, 128 or 256 query rows of one sequence, query head); each
+// wave owns 32 rows. The block-table entries of the key range go to LDS once. K and V tiles of 64 keys are gathered from the pages into LDS for all
 // waves (the next tile's 16-byte chunks already in flight in registers);
 // S^T = K Q^T and O^T += V^T P^T run on v_mfma_f32_32x32x16_bf16 with the query
 // on the MFMA lane, so the online softmax is in-register. Tiles that lie wholly
@@ -660,13 +660,17 @@ __global__ __launch_bounds__(64 * WM_WAVES) void window_attn_mfma_kernel(WinAttn
 
 int window_attention_mfma(const WinAttnParams& p, int max_q, hipStream_t st) {
   if (max_q <= 0) return 0;
-  // 128-row blocks when they alone fill the GPU several times over, else 64-row blocks
-  const long wg4 = (long)((max_q + 127) / 128) * p.H * p.B;
-  const int waves = wg4 >= 1024 ? 4 : 2;
+  // the widest row block the longest feed fills: the tiles' staging (gather
+  // through the page table, LDS stores, barriers) is paid once per block and
+  // tile, and measured times fall with the block width even when the grid
+  // shrinks below the number of compute units
+  const int waves = max_q > 128 ? 8 : (max_q > 64 ? 4 : 2);
   const dim3 grid((max_q + waves * 32 - 1) / (waves * 32), p.H, p.B);
 #define GO(A, C)                                                                              \
   if (p.D == A && p.Dv == C) {                                                                \
-    if (waves == 4)                                                                           \
+    if (waves == 8)                                                                           \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<A, C, 8>), grid, dim3(512), 0, st, p);      \
+    else if (waves == 4)                                                                      \
       hipLaunchKernelGGL((window_attn_mfma_kernel<A, C, 4>), grid, dim3(256), 0, st, p);      \
     else                                                                                      \
       hipLaunchKernelGGL((window_attn_mfma_kernel<A, C, 2>), grid, dim3(128), 0, st, p);      \
