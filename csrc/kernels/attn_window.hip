@@ -24,21 +24,29 @@
 // serves REP query heads of the group at once, so K and V are read once per
 // group. The visible keys go in 64-key windows aligned to multiples of 64
 // positions, one per wave in turn (window index modulo the wave count; 16 waves
-// when the launch has few workgroups, else 4): scores
-// with a lane per key, an online softmax per head across the wave, values with
-// a lane per output column. The waves' partial (max, sum, accumulator) triples
-// merge through LDS in wave order. Which windows a wave takes and the order of
-// every sum depend only on the query's position and the wave count. When a
-// step has few rows and long contexts the windows are also dealt out to several
-// workgroups per row, whose partial triples a small combine launch merges.
+// when the launch has few workgroups, else 4). In a window, groups of D / 8
+// lanes (D / 4 for f32) cover a key row in 16-byte runs, so one load brings
+// whole rows; a lane multiplies its run with its part of q in registers, the
+// group adds up with data-parallel moves, and one lane of the group keeps the
+// key's score. An online softmax per head runs across the wave; the value rows
+// are read in the same 16-byte runs, a lane sums its run over the rows of its
+// group, and the groups are added once at the end. (Head sizes that are no
+// power-of-two number of runs: a lane per key, a lane per output column.) The
+// waves' partial (max, sum, accumulator) triples merge through LDS in wave
+// order. Which windows a wave takes and the order of every sum depend only on
+// the query's position and the wave count. When a step has few rows and long
+// contexts the windows are also dealt out to several workgroups per row, whose
+// partial triples a small combine launch merges.
 //
 // window_attn_mfma_kernel (bf16, D and Dv in {64, 128}; prompt portions): a
 // workgroup per (64, 128 or 256 query rows of one sequence, query head); each
-// wave owns 32 rows. The block-table entries of the key range go to LDS once. K and V tiles of 64 keys are gathered from the pages into LDS for all
-// waves (the next tile's 16-byte chunks already in flight in registers);
+// wave owns 32 rows. The block-table entries of the key range go to LDS once.
+// K and V tiles of 64 keys are gathered from the pages into LDS for all waves
+// (the next tile's 16-byte chunks already in flight in registers);
 // S^T = K Q^T and O^T += V^T P^T run on v_mfma_f32_32x32x16_bf16 with the query
 // on the MFMA lane, so the online softmax is in-register. Tiles that lie wholly
-// between the kept first tokens and the rows' windows are skipped.
+// between the kept first tokens and the rows' windows are skipped, and a tile
+// that every row of a wave sees whole takes a path without per-score tests.
 #include "seqmix.h"
 
 struct WinAttnParams {

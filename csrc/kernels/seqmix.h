@@ -1,5 +1,6 @@
 // Helpers shared by the sequence-mixer kernels of the hybrid decoders
-// (norm_dyt.hip, attn_latent.hip, lightning.hip, moe.hip).
+// (norm_dyt.hip, attn_latent.hip, lightning.hip, moe.hip, seq_rows.hip,
+// attn_sigmoid.hip, norm_scalar.hip, norm_rms1p.hip, attn_window.hip, mamba2.hip).
 //
 // Activations are bfloat16 or float32, chosen at run time by a dtype code
 // (0: bf16, 1: f32); every kernel is a template over the storage type and does

@@ -1,12 +1,18 @@
 """Entry points of the sequence-mixer ops of the hybrid decoders: Dynamic-Tanh
 norm, latent (compressed-KV) attention with a softmax sink over a paged latent
 cache, decayed linear attention with a carried per-sequence state, and the
-grouped top-k expert router with its expert feed-forward.
+grouped top-k expert router with its expert feed-forward; further down the
+row-state ops and sigmoid attention of the Sodonex family, and the pre-norm /
+layer-scale residual step, windowed softmax attention over paged K / V and the
+Mamba-2 input stage of the Movinex family (whose recurrence is ``state_scan``,
+the generalised lightning scan).
 
 As everywhere in ``ops``: GPU tensors run the HIP kernels
 (``csrc/kernels/norm_dyt.hip``, ``attn_latent.hip``, ``lightning.hip``,
-``moe.hip``), CPU tensors the f32 PyTorch references (the CPU test tier and the
-numerics oracle of the GPU tests). Activations are bfloat16 or float32
+``moe.hip``, ``seq_rows.hip``, ``attn_sigmoid.hip``, ``norm_scalar.hip``,
+``norm_rms1p.hip``, ``attn_window.hip``, ``mamba2.hip``), CPU tensors the f32
+PyTorch references (the CPU test tier and the numerics oracle of the GPU
+tests). Activations are bfloat16 or float32
 (``_DT``); the residual stream, scores, softmax, recurrent state, router and
 norm statistics are f32 in both.
 """
