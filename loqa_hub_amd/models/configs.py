@@ -490,15 +490,20 @@ def movinex_config_from_json(d: dict, name: str = "movinex") -> MovinexConfig:
     for i, L in enumerate(d["layers"]):
         m, kind = L["mixer"], L["type"]
         if kind in ("attention", "attention_2"):
+            # the two kinds differ in what they have at all: the first one biases,
+            # a value projection and the query temperature; the second one rotary
+            # positions, the soft cap, the window with kept tokens and the gate
             second = kind == "attention_2"
-            r, qt, mk = m.get("rot"), m.get("q_temp"), m.get("mask") or {}
+            r = m.get("rot") if second else None
+            qt = None if second else m.get("q_temp")
+            mk = (m.get("mask") or {}) if second else {}
             mixer = SoftmaxAttnConfig(
                 int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m.get("vdim", m["dim"])),
                 float(m["scale"]), bias=not second, values_from_keys=second, gate=second,
                 rot=RotaryConfig(int(r["dims"]), float(r["base"])) if r else None,
                 q_temp=(float(qt["coef"]), int(qt["every"])) if qt else None,
-                softcap=float(m.get("softcap") or 0.0), window=int(mk.get("size") or 0),
-                keep_first=int(mk.get("keep_first") or 0))
+                softcap=float(m.get("softcap") or 0.0) if second else 0.0,
+                window=int(mk.get("size") or 0), keep_first=int(mk.get("keep_first") or 0))
             if mixer.heads % mixer.kv_heads:
                 raise ValueError(f"layer {i}: {mixer.heads} heads do not split over "
                                  f"{mixer.kv_heads} key/value heads")
