@@ -225,6 +225,9 @@ class RotaryConfig:
     dims: int                       # rotated entries (pairs 2i, 2i+1), <= rot_dim
     base: float
     yarn: tuple | None = None       # (factor, original, fast, slow)
+    # the checkpoint pairs entry i with entry i + dims / 2 (rotate-half layout);
+    # a loader may fold this into the interleaved layout by permuting rows
+    half: bool = False
 
 
 @dataclass(frozen=True)
@@ -237,6 +240,8 @@ class LatentAttnConfig:
     scale: float
     rot: RotaryConfig
     kv_from: int | None = None      # reuse that layer's latent cache
+    q_rank: int = 0                 # > 0: queries go through an RMS-normed latent of this size
+    gate: bool = False              # heads' outputs times sigmoid(W_g h), per entry
 
 
 @dataclass(frozen=True)
@@ -431,6 +436,11 @@ class SoftmaxAttnConfig:
     softcap: float = 0.0            # score <- cap tanh(score / cap); 0: none
     window: int = 0                 # key j visible if p - j < window ...; 0: every earlier key
     keep_first: int = 0             # ... or j < keep_first
+    # "head": q and k divided by their root mean square per head after rotation,
+    # no weight; "whole": RMS norm over the whole q (and k) projection with a
+    # weight vector of that size, before rotation
+    qk_norm: str = "head"
+    zero_sink: bool = False         # the softmax denominator holds one more term exp(0)
 
 
 @dataclass(frozen=True)
@@ -551,3 +561,130 @@ def movinex_config_from_json(d: dict, name: str = "movinex") -> MovinexConfig:
             loop = None
     return MovinexConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
                          float(d.get("logit_scale", 1.0)), tuple(layers), loop)
+
+
+# --------------------------------------------------------------------------
+# Vilulix: a decoder of parallel layers, x <- x + mixer(norm1(x)) + ff(norm2(x))
+# with both RMS norms (weights stored around zero) reading the same x. A
+# stretch of layers may run several times in a row with the same weights, the
+# embedding output added to x before every pass but the first. Mixers: a
+# stabilised matrix memory with exponential gates (mLSTM), latent attention
+# with a query latent and an output gate, and a pair of mixers side by side -
+# sliding-window softmax attention with a zero sink beside a gated delta rule
+# with short convolutions. Dense SwiGLU feed-forwards; the logits are
+# soft-capped. Every size and constant comes from config.json or a tensor's
+# shape.
+@dataclass(frozen=True)
+class MatrixMemoryConfig:
+    heads: int
+    dim: int                        # query / key size per head
+    vdim: int
+    gate_cap: float                 # gate pre-activations pass cap tanh(z / cap)
+
+
+@dataclass(frozen=True)
+class DeltaRuleConfig:
+    heads: int                      # value heads
+    kv_heads: int                   # query / key heads shared by heads / kv_heads neighbours
+    dim: int
+    vdim: int
+    taps: int                       # short causal convolution on q, k and v
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+
+@dataclass(frozen=True)
+class ParallelMixerConfig:
+    left: SoftmaxAttnConfig
+    right: DeltaRuleConfig
+    left_scale: float
+    right_scale: float
+
+
+@dataclass(frozen=True)
+class VilulixConfig:
+    name: str
+    vocab_size: int
+    d_model: int
+    norm_eps: float
+    logit_softcap: float            # 0: none
+    layers: tuple
+    loop: LoopConfig | None = None
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list[tuple[int, bool]]:
+        """The layers in execution order as (layer index, first of a LATER pass
+        of the repeated stretch: the embedding output is added before it);
+        every run has a cache or state of its own."""
+        n = len(self.layers)
+        if self.loop is None:
+            return [(i, False) for i in range(n)]
+        lp = self.loop
+        out = [(i, False) for i in range(lp.start)]
+        for t in range(lp.times):
+            out += [(i, t > 0 and i == lp.start) for i in range(lp.start, lp.stop)]
+        return out + [(i, False) for i in range(lp.stop, n)]
+
+
+def _rot_half(r: dict, size: int, where: str) -> RotaryConfig:
+    rot = RotaryConfig(int(r["dims"]), float(r["base"]), half=True)
+    if rot.dims % 2 or not 0 <= rot.dims <= size:
+        raise ValueError(f"{where}: rot.dims {rot.dims} does not fit {size} entries")
+    return rot
+
+
+def vilulix_config_from_json(d: dict, name: str = "vilulix") -> VilulixConfig:
+    layers = []
+    for i, L in enumerate(d["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind == "mlstm":
+            mixer = MatrixMemoryConfig(int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                                       float(m["gate_cap"]))
+            if mixer.gate_cap <= 0:
+                raise ValueError(f"layer {i}: gate_cap must be positive")
+        elif kind == "latent_attention":
+            mixer = LatentAttnConfig(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]),
+                                     int(m["vdim"]), int(m["kv_rank"]), float(m["scale"]),
+                                     _rot_half(m["rot"], int(m["rot_dim"]), f"layer {i}"),
+                                     q_rank=int(m["q_rank"]), gate=True)
+            if mixer.q_rank < 1 or mixer.kv_rank < 1:
+                raise ValueError(f"layer {i}: latent sizes must be positive")
+        elif kind == "parallel":
+            a, r = m["left"], m["right"]
+            left = SoftmaxAttnConfig(int(a["heads"]), int(a["kv_heads"]), int(a["dim"]),
+                                     int(a["vdim"]), float(a["scale"]),
+                                     rot=_rot_half(a["rot"], int(a["dim"]), f"layer {i}"),
+                                     window=int(a["mask"]["size"]), qk_norm="whole", zero_sink=True)
+            right = DeltaRuleConfig(int(r["heads"]), int(r["kv_heads"]), int(r["dim"]),
+                                    int(r["vdim"]), int(r["conv"]))
+            if left.heads % left.kv_heads or right.heads % right.kv_heads:
+                raise ValueError(f"layer {i}: heads do not split over the key/value heads")
+            if left.window < 1 or right.taps < 1:
+                raise ValueError(f"layer {i}: mask size and conv taps must be positive")
+            mixer = ParallelMixerConfig(left, right, float(m["left_scale"]),
+                                        float(m["right_scale"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = L.get("mlp")
+        if not f:
+            mlp = None
+        elif f["kind"] == "dense":
+            mlp = FeedForwardConfig("dense", int(f["ff"]))
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(HybridLayerConfig(kind, mixer, mlp))
+    lp = d.get("loop")
+    loop = None
+    if lp:
+        loop = LoopConfig(int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+        if not 0 <= loop.start <= loop.stop <= len(layers) or loop.times < 1:
+            raise ValueError("loop: start, stop and times do not fit the layer list")
+        if loop.start == loop.stop or loop.times == 1:
+            loop = None
+    return VilulixConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
+                         float(d.get("logit_softcap") or 0.0), tuple(layers), loop)

@@ -488,3 +488,20 @@ def save_movinex(cfg, state: dict[str, torch.Tensor], folder: str) -> None:
     write_safetensors(state, os.path.join(folder, "model.safetensors"))
     with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as f:
         json.dump(config_to_json(cfg), f, indent=1)
+
+
+def load_vilulix(cfg, path: str, device, dtype=torch.bfloat16, max_positions: int = 8192):
+    """A Vilulix checkpoint (its own tensor naming) in the fused device layout;
+    ``dtype`` is the activation / matrix dtype (bfloat16 serving, float32 exact)."""
+    from .vilulix import VilulixWeights
+    return VilulixWeights(cfg, read_safetensors_raw(path), device, dtype, max_positions)
+
+
+def save_vilulix(cfg, state: dict[str, torch.Tensor], folder: str) -> None:
+    """Write ``state`` (checkpoint naming) and the config.json of ``cfg``."""
+    import json
+    from .vilulix import config_to_json
+    os.makedirs(folder, exist_ok=True)
+    write_safetensors(state, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(config_to_json(cfg), f, indent=1)

@@ -38,6 +38,74 @@ from ..ops.seqmix import DytParams
 from .configs import PipizenConfig
 
 
+def latent_prompt_layout(L: dict, m, dtype, device) -> None:
+    """Padded per-head copies for the matrix-core prompt kernel (bf16): the
+    query projection ``wq`` with DKp rows per head, W_uk / W_uv producing [H,
+    DKp] keys and [H, DVp] values from a latent row, and W_o with DVp columns
+    per head. Sizes that the kernel is built for are used as they are. ``L``
+    holds ``wq`` [H (D + Dr), n], ``wuk`` [H, D, R], ``wuv_t`` [H, R, Dv] and
+    ``wo``; shared by every family with latent attention layers."""
+    H, D, Dr, Dv, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
+    sizes = seqmix.prefill_head_sizes(D + Dr, Dv) if dtype == torch.bfloat16 else None
+    if sizes is None or torch.device(device).type != "cuda":
+        return
+    DKp, DVp = sizes
+    dev, dt = device, dtype
+
+    def pad_rows(w, per, to):       # [H * per, n] -> [H * to, n], zero rows after each head
+        if per == to:
+            return w
+        out = torch.zeros(H, to, w.shape[1], dtype=dt, device=dev)
+        out[:, :per] = w.view(H, per, -1)
+        return out.view(H * to, -1).contiguous()
+    L["wq"], L["qw"] = pad_rows(L["wq"], D + Dr, DKp), DKp
+    L["wuk_p"] = pad_rows(L["wuk"].reshape(H * D, R), D, DKp)
+    L["wuv_p"] = pad_rows(L["wuv_t"].transpose(1, 2).reshape(H * Dv, R), Dv, DVp)
+    L["wo_p"] = L["wo"] if DVp == Dv else \
+        pad_rows(L["wo"].t().contiguous(), Dv, DVp).t().contiguous()
+    L["prompt_sizes"] = (DKp, DVp)
+
+
+def latent_mix(L: dict, m, q: torch.Tensor, z: torch.Tensor | None, pages: torch.Tensor, meta,
+               eps: float, prompt_min_q: int, gate: torch.Tensor | None = None) -> torch.Tensor:
+    """Latent attention of one step after its projections, for every family
+    that has such layers. q [T, H * qw]: the projected queries (per head D
+    unrotated then Dr rotary entries, possibly padded to ``L["qw"]``); z [T, R +
+    Dr]: the projected latent and shared rotary key part, appended to ``pages``
+    here (None: the pages belong to another layer and are complete). ``gate``
+    [T, H Dv] multiplies the heads' outputs by sigmoid(gate) before the output
+    projection. Returns the mixer's output [T, width]."""
+    H, D, Dr, Dv, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
+    T = q.shape[0]
+    if z is not None:
+        seqmix.latent_append(z, L["dkv_norm"], eps, meta.positions, L["cos_sin"], pages,
+                             meta.slots, R, m.rot.dims)
+    q = q.view(T, H, L["qw"])
+    if "prompt_sizes" in L and meta.max_q >= prompt_min_q and meta.cu_k is not None:
+        # prompt pass: per-head keys / values from the gathered latents, then
+        # flash attention on the matrix cores
+        DKp, DVp = L["prompt_sizes"]
+        cl, kr = seqmix.latent_gather(pages, meta.block_tables, meta.cu_k, meta.total_k,
+                                      meta.max_ctx, R)
+        k = ops.linear(cl, L["wuk_p"]).view(-1, H, DKp)
+        seqmix.latent_kfill_(k, kr, D)
+        v = ops.linear(cl, L["wuv_p"]).view(-1, H, DVp)
+        seqmix.rope_pairs_(q, D, m.rot.dims, meta.positions, L["cos_sin"])
+        o = seqmix.latent_prefill(q, k, v, meta.cu_q, meta.cu_k, meta.positions, L["sink"],
+                                  m.scale, meta.max_q)
+        if gate is not None:
+            seqmix.sigmoid_gate_(o.view(T, H, DVp), gate, H, Dv)
+        return ops.linear(o, L["wo_p"])
+    qa = torch.bmm(q[:, :, :D].transpose(0, 1), L["wuk"])            # [H, T, R]
+    lat = seqmix.latent_attention(qa, q[:, :, D:D + Dr], pages, meta.cu_q, meta.ctx_lens,
+                                  meta.block_tables, meta.positions, L["cos_sin"], L["sink"],
+                                  m.scale, R, m.rot.dims, meta.max_ctx)
+    o = torch.bmm(lat, L["wuv_t"]).transpose(0, 1).reshape(T, H * Dv)     # [T, H Dv]
+    if gate is not None:
+        seqmix.sigmoid_gate_(o.view(T, H, Dv), gate, H, Dv)
+    return ops.linear(o, L["wo"])
+
+
 class PipizenWeights:
     """Device weights in the fused layouts, from a state dict in checkpoint
     naming (``embed``, ``l<i>.norm1[.b|.alpha]``, ``l<i>.mix.*``, ``l<i>.mlp.*``,
@@ -111,29 +179,7 @@ class PipizenWeights:
             self.layers.append(L)
 
     def _prompt_layout(self, L: dict, m) -> None:
-        """Padded per-head copies for the matrix-core prompt kernel (bf16): the
-        query projection with DKp rows per head, W_uk / W_uv producing [H, DKp]
-        keys and [H, DVp] values from a latent row, and W_o with DVp columns per
-        head. Sizes that the kernel is built for are used as they are."""
-        H, D, Dr, Dv, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
-        sizes = seqmix.prefill_head_sizes(D + Dr, Dv) if self.dtype == torch.bfloat16 else None
-        if sizes is None or self.device.type != "cuda":
-            return
-        DKp, DVp = sizes
-        dev, dt = self.device, self.dtype
-
-        def pad_rows(w, per, to):       # [H * per, n] -> [H * to, n], zero rows after each head
-            if per == to:
-                return w
-            out = torch.zeros(H, to, w.shape[1], dtype=dt, device=dev)
-            out[:, :per] = w.view(H, per, -1)
-            return out.view(H * to, -1).contiguous()
-        L["wq"], L["qw"] = pad_rows(L["wq"], D + Dr, DKp), DKp
-        L["wuk_p"] = pad_rows(L["wuk"].reshape(H * D, R), D, DKp)
-        L["wuv_p"] = pad_rows(L["wuv_t"].transpose(1, 2).reshape(H * Dv, R), Dv, DVp)
-        L["wo_p"] = L["wo"] if DVp == Dv else \
-            pad_rows(L["wo"].t().contiguous(), Dv, DVp).t().contiguous()
-        L["prompt_sizes"] = (DKp, DVp)
+        latent_prompt_layout(L, m, self.dtype, self.device)
 
     def _table(self, rot) -> torch.Tensor:
         key = (rot.dims, rot.base, rot.yarn)
@@ -295,33 +341,10 @@ class PipizenModel:
         return ops.linear(hf, w.head)
 
     def _latent(self, i, m, L, h, meta, cache, T) -> torch.Tensor:
-        H, D, Dr, Dv, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
         src = i if m.kv_from is None else m.kv_from
-        pages = cache.latent[src]
-        if m.kv_from is None:
-            z = ops.linear(h, L["wdkv"])
-            seqmix.latent_append(z, L["dkv_norm"], self.cfg.norm_eps, meta.positions, L["cos_sin"],
-                                 pages, meta.slots, R, m.rot.dims)
-        q = ops.linear(h, L["wq"]).view(T, H, L["qw"])
-        if "prompt_sizes" in L and meta.max_q >= self.prompt_min_q and meta.cu_k is not None:
-            # prompt pass: per-head keys / values from the gathered latents, then
-            # flash attention on the matrix cores
-            DKp, DVp = L["prompt_sizes"]
-            cl, kr = seqmix.latent_gather(pages, meta.block_tables, meta.cu_k, meta.total_k,
-                                          meta.max_ctx, R)
-            k = ops.linear(cl, L["wuk_p"]).view(-1, H, DKp)
-            seqmix.latent_kfill_(k, kr, D)
-            v = ops.linear(cl, L["wuv_p"]).view(-1, H, DVp)
-            seqmix.rope_pairs_(q, D, m.rot.dims, meta.positions, L["cos_sin"])
-            o = seqmix.latent_prefill(q, k, v, meta.cu_q, meta.cu_k, meta.positions, L["sink"],
-                                      m.scale, meta.max_q)
-            return ops.linear(o, L["wo_p"])
-        qa = torch.bmm(q[:, :, :D].transpose(0, 1), L["wuk"])            # [H, T, R]
-        lat = seqmix.latent_attention(qa, q[:, :, D:D + Dr], pages, meta.cu_q, meta.ctx_lens,
-                                      meta.block_tables, meta.positions, L["cos_sin"], L["sink"],
-                                      m.scale, R, m.rot.dims, meta.max_ctx)
-        o = torch.bmm(lat, L["wuv_t"])                                    # [H, T, Dv]
-        return ops.linear(o.transpose(0, 1).reshape(T, H * Dv), L["wo"])
+        z = ops.linear(h, L["wdkv"]) if m.kv_from is None else None
+        return latent_mix(L, m, ops.linear(h, L["wq"]), z, cache.latent[src], meta,
+                          self.cfg.norm_eps, self.prompt_min_q)
 
     def _lightning(self, i, m, L, h, meta, cache) -> torch.Tensor:
         H, D, Dv = m.heads, m.dim, m.vdim

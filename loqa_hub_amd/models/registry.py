@@ -3,7 +3,8 @@ config.json: the Llama family (Hugging Face naming) and the designs with their
 own naming, told apart by ``"architecture"``: the hybrid Pipizen (latent /
 lightning mixers), Sodonex (chunked sigmoid attention with row state) and
 Movinex (windowed softmax attention, Mamba-2 layers, a repeated stretch of
-layers). A family knows how to
+layers) and Vilulix (parallel layers; matrix memory, latent attention, windowed
+attention beside a gated delta rule). A family knows how to
 read its config, load or seed its weights and build its step function; the
 engine, the scheduler and the command line go through this table only.
 """
@@ -14,9 +15,10 @@ from typing import Callable
 
 import torch
 
-from .configs import (LlamaConfig, MovinexConfig, PipizenConfig, SodonexConfig, checkpoint_config,
-                      llama_config_from_hf, movinex_config_from_json, pipizen_config_from_json,
-                      sodonex_config_from_json)
+from .configs import (LlamaConfig, MovinexConfig, PipizenConfig, SodonexConfig, VilulixConfig,
+                      checkpoint_config, llama_config_from_hf, movinex_config_from_json,
+                      pipizen_config_from_json, sodonex_config_from_json,
+                      vilulix_config_from_json)
 
 
 @dataclass(frozen=True)
@@ -40,6 +42,10 @@ def _is_movinex(d: dict) -> bool:
     return str(d.get("architecture", "")).lower() == "movinex"
 
 
+def _is_vilulix(d: dict) -> bool:
+    return str(d.get("architecture", "")).lower() == "vilulix"
+
+
 def _is_llama(d: dict) -> bool:
     arch = " ".join(d.get("architectures") or []) + " " + str(d.get("model_type", ""))
     return "num_attention_heads" in d and ("llama" in arch.lower() or "hidden_size" in d)
@@ -49,6 +55,7 @@ FAMILIES = (
     Family("pipizen", PipizenConfig, _is_pipizen, pipizen_config_from_json, True),
     Family("sodonex", SodonexConfig, _is_sodonex, sodonex_config_from_json, True),
     Family("movinex", MovinexConfig, _is_movinex, movinex_config_from_json, True),
+    Family("vilulix", VilulixConfig, _is_vilulix, vilulix_config_from_json, True),
     Family("llama", LlamaConfig, _is_llama, llama_config_from_hf, False),
 )
 
@@ -91,6 +98,8 @@ def load_lm_weights(cfg, path: str, device, *, dtype=torch.bfloat16, tp=None,
         return loader.load_sodonex(cfg, path, device, dtype, max_positions)
     if fam.name == "movinex":
         return loader.load_movinex(cfg, path, device, dtype, max_positions)
+    if fam.name == "vilulix":
+        return loader.load_vilulix(cfg, path, device, dtype, max_positions)
     return loader.load_pipizen(cfg, path, device, dtype, max_positions)
 
 
@@ -106,6 +115,9 @@ def random_lm_weights(cfg, device, *, seed: int = 0, dtype=torch.bfloat16, tp=No
     if fam.name == "movinex":
         from .movinex import MovinexWeights
         return MovinexWeights.random(cfg, device, seed, dtype, max_positions)
+    if fam.name == "vilulix":
+        from .vilulix import VilulixWeights
+        return VilulixWeights.random(cfg, device, seed, dtype, max_positions)
     from .pipizen import PipizenWeights
     return PipizenWeights.random(cfg, device, seed, dtype, max_positions)
 
@@ -120,5 +132,8 @@ def build_model(weights):
     from .movinex import MovinexModel, MovinexWeights
     if isinstance(weights, MovinexWeights):
         return MovinexModel(weights)
+    from .vilulix import VilulixModel, VilulixWeights
+    if isinstance(weights, VilulixWeights):
+        return VilulixModel(weights)
     from .pipizen import PipizenModel
     return PipizenModel(weights)

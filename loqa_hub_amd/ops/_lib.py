@@ -237,11 +237,23 @@ _SEQMIX_SIGS = {
     "loqa_rms1p_norm": [_vp, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
     "loqa_scaled_add_rms1p": [_vp, _vp, _i, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
     "loqa_qk_prep_append": [_vp, _i, _l, _i, _i, _i, _i, _i, _vp, _i, _i, _f, _f, _i, _vp, _vp,
-                            _vp, _i, _i, _vp, _vp, _i, _vp],
+                            _vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp],
     "loqa_window_attention": [_vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _l, _f, _f,
-                              _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp],
+                              _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp],
     "loqa_mamba2_prep": [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp,
                          _vp, _i, _i, _vp, _vp, _vp],
+    "loqa_residual_rms1p": [_vp, _vp, _f, _vp, _f, _vp, _f, _i, _vp, _vp, _vp, _f, _vp, _vp, _i,
+                            _i, _i, _vp],
+    "loqa_rms_norm_cols": [_vp, _i, _l, _i, _vp, _f, _vp, _i, _i, _vp],
+    "loqa_sigmoid_gate": [_vp, _i, _vp, _l, _i, _i, _i, _i, _vp],
+    "loqa_softcap": [_vp, _l, _f, _vp],
+    "loqa_exp_gate_scan": [_vp, _i, _vp, _vp, _f, _vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp],
+    "loqa_matrix_memory_inputs": [_vp, _i, _l, _i, _i, _i, _vp, _i, _vp],
+    "loqa_normalized_gated_rmsnorm": [_vp, _vp, _vp, _vp, _i, _l, _f, _vp, _i, _i, _i, _i, _vp],
+    "loqa_delta_prep": [_vp, _i, _l, _vp, _i, _i, _i, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp,
+                        _vp, _i, _i, _vp, _vp, _vp],
+    "loqa_delta_scan": [_vp, _l, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i,
+                        _i, _vp],
 }
 _seqmix = None
 

@@ -758,10 +758,12 @@ def lightning_scan(qkv, H: int, D: int, Dv: int, state, state_slots, cu_q, posit
                       decay=decay)
 
 
-def gated_rmsnorm(o, w, gate, eps: float, out_dtype, groups: int = 1, silu_first: bool = False):
-    """rmsnorm(o) * w * sigmoid(gate), the row normalised as a whole; with
-    ``silu_first``: rmsnorm(o * silu(gate)) * w (the gate before the norm).
-    ``groups`` > 1 normalises the row in that many equal parts."""
+def gated_rmsnorm(o, w, gate, eps: float, out_dtype, groups: int = 1, silu_first: bool = False,
+                  gate_act: str = "sigmoid"):
+    """rmsnorm(o) * w * sigmoid(gate), the row normalised as a whole (``gate_act``
+    "silu": times silu(gate) instead); with ``silu_first``: rmsnorm(o *
+    silu(gate)) * w (the gate before the norm). ``groups`` > 1 normalises the
+    row in that many equal parts."""
     of, g = o.float(), gate.float()
     T, n = of.shape
     if silu_first:
@@ -769,7 +771,7 @@ def gated_rmsnorm(o, w, gate, eps: float, out_dtype, groups: int = 1, silu_first
     y = of.view(T, groups, n // groups)
     y = (y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)).view(T, n) * w.float()
     if not silu_first:
-        y = y * torch.sigmoid(g)
+        y = y * (torch.sigmoid(g) if gate_act == "sigmoid" else torch.nn.functional.silu(g))
     return y.to(out_dtype)
 
 
@@ -1004,7 +1006,7 @@ def scaled_add_rms1p(resid, y, ls, nxt, eps: float, out_dtype):
 
 
 def qk_prep_append(u, H: int, G: int, D: int, Dv: int, v_off: int, cos_sin, dims: int, eps: float,
-                   q_temp, positions, k_cache, v_cache, slots, out_dtype):
+                   q_temp, positions, k_cache, v_cache, slots, out_dtype, q_norm=None, k_norm=None):
     """u [T, >= H D + G D (+ G Dv)]: projected q | k (| v) rows. Per head: the
     first ``dims`` entries of q and k rotate pairwise (2i with 2i + 1) by the
     position's angles, then each head's q and k is divided by its root mean
@@ -1012,18 +1014,25 @@ def qk_prep_append(u, H: int, G: int, D: int, Dv: int, v_off: int, cos_sin, dims
     temperature 1 + coef ln(floor((p + 1) / every) + 1) when ``q_temp`` =
     (coef, every). k goes to its pages [blocks, BLK, G D]; the value rows - the
     columns at ``v_off``, or with ``v_off`` < 0 the k columns as projected - go to
-    theirs [blocks, BLK, G Dv] at ``slots`` (-1: padding row). Returns q [T, H D]."""
+    theirs [blocks, BLK, G Dv] at ``slots`` (-1: padding row). Returns q [T, H D].
+    With ``q_norm`` [H D] and ``k_norm`` [G D] the norm is another one: q and k
+    are RMS-normed over their whole projection with these weights BEFORE the
+    rotation, and no per-head division follows."""
     T = u.shape[0]
     uf = u.float()
     q = uf[:, :H * D].reshape(T, H, D)
     k = uf[:, H * D:(H + G) * D].reshape(T, G, D)
     v = k.reshape(T, G * D) if v_off < 0 else uf[:, v_off:v_off + G * Dv]
     pos = positions[:T].long()
+    if q_norm is not None:
+        q = rms_norm_cols(q.reshape(T, H * D), H * D, q_norm, eps, torch.float32).view(T, H, D)
+        k = rms_norm_cols(k.reshape(T, G * D), G * D, k_norm, eps, torch.float32).view(T, G, D)
     if dims:
         cs = cos_sin[pos]
         q, k = rotate_pairs(q, cs, dims), rotate_pairs(k, cs, dims)
-    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
-    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+    if q_norm is None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
     if q_temp is not None:
         coef, every = q_temp
         steps = torch.div(pos + 1, int(every), rounding_mode="floor").float()
@@ -1038,12 +1047,14 @@ def qk_prep_append(u, H: int, G: int, D: int, Dv: int, v_off: int, cos_sin, dims
 
 def window_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions, scale: float,
                      softcap: float, window: int, keep_first: int, gate, H: int, G: int, D: int,
-                     Dv: int, out_dtype):
+                     Dv: int, out_dtype, sink=None):
     """Softmax attention of q [T, H D] over paged K [blocks, BLK, G D] and V
     [blocks, BLK, G Dv]: score = q . k * scale, soft-capped to cap tanh(score /
     cap) when ``softcap`` > 0; a query at position p sees key j <= p, and with
     ``window`` > 0 only if p - j < window or j < keep_first. ``gate`` [T, H Dv]
-    multiplies the output by sigmoid(gate) per entry. Returns [T, H Dv]."""
+    multiplies the output by sigmoid(gate) per entry. ``sink`` f32 [H]: the
+    softmax denominator of head h also holds exp(sink[h]), a term without a
+    value. Returns [T, H Dv]."""
     T = q.shape[0]
     blk = k_cache.shape[1]
     rep = H // G
@@ -1068,7 +1079,9 @@ def window_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, position
             if softcap > 0:
                 s = softcap * torch.tanh(s / softcap)
             s = s.masked_fill(~seen, float("-inf"))
-            out[q0:q1, h] = torch.softmax(s, dim=-1) @ vv[:, h // rep]
+            if sink is not None:
+                s = torch.cat([s, sink[h].float().expand(q1 - q0, 1)], dim=-1)
+            out[q0:q1, h] = torch.softmax(s, dim=-1)[:, :L] @ vv[:, h // rep]
     out = out.view(T, H * Dv)
     if gate is not None:
         out = out * torch.sigmoid(gate.float())
@@ -1106,3 +1119,174 @@ def mamba2_prep(u, x_off: int, C: int, dt_off: int, Hh: int, conv_w, conv_b, dt_
     y = torch.nn.functional.silu(y + conv_b.float())
     dt = torch.nn.functional.softplus(u[:, dt_off:dt_off + Hh].float() + dt_bias.float())
     return y, torch.stack([torch.exp(a_neg.float() * dt), dt], dim=-1).contiguous()
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of decoders with parallel layers (models/vilulix.py): the
+# residual step that adds several sublayer outputs at once and norms the sum
+# twice, the gate scan and input stage of a stabilised matrix memory, the
+# input stage and recurrence of a gated delta rule, a plain RMS norm over a
+# column slice, an output gate and the soft cap of the logits.
+def residual_rms1p(resid, addends, extra, w_a, w_b, eps: float, out_dtype):
+    """resid (f32, in place) += sum_i scale_i * y_i (+ ``extra``, f32); returns
+    (rms1p_norm(resid; w_a), rms1p_norm(resid; w_b)), None where the weight is
+    None. ``addends``: up to three (tensor, scale)."""
+    for y, s in addends:
+        resid.add_(y.float() * float(s))
+    if extra is not None:
+        resid.add_(extra.float())
+    return (None if w_a is None else rms1p_norm(resid, w_a, eps, out_dtype),
+            None if w_b is None else rms1p_norm(resid, w_b, eps, out_dtype))
+
+
+def rms_norm_cols(u, n: int, w, eps: float, out_dtype):
+    """RMS norm with a plain weight over the first ``n`` columns of u [T, >= n]."""
+    x = u[:, :n].float()
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def sigmoid_gate_(o, gate, H: int, Dv: int):
+    """o [T, H, Dvo >= Dv] (in place): the first Dv entries of every head times
+    sigmoid(gate [T, H Dv])."""
+    T = o.shape[0]
+    g = torch.sigmoid(gate.float()).view(T, H, Dv)
+    o[:, :, :Dv] = (o[:, :, :Dv].float() * g).to(o.dtype)
+    return o
+
+
+def softcap_(x, cap: float):
+    """x <- cap tanh(x / cap) in place (f32)."""
+    return x.copy_(cap * torch.tanh(x / cap))
+
+
+def exp_gate_scan(gz, i_bias, f_bias, cap: float, m_state, state_slots, cu_q, positions):
+    """The gates of a stabilised exponential-gate memory over a flat token
+    batch. gz f32 [T, 2 H]: pre-activations of the input gates (first H
+    columns) and the forget gates. Per head: li = cap tanh((z_i + b_i) / cap),
+    lf = logsigmoid(cap tanh((z_f + b_f) / cap)), running maximum m_t =
+    max(lf + m_{t-1}, li) (m = 0 before position 0, else ``m_state[slot]``).
+    Returns tok f32 [T, H, 2] = (exp(lf + m_{t-1} - m_t), exp(li - m_t)) and
+    floor f32 [T, H] = exp(-m_t); ``m_state`` [slots, H] takes the last m."""
+    T = gz.shape[0]
+    H = gz.shape[1] // 2
+    z = gz.float()
+    li = cap * torch.tanh((z[:, :H] + i_bias.float()) / cap)
+    lf = torch.nn.functional.logsigmoid(cap * torch.tanh((z[:, H:] + f_bias.float()) / cap))
+    tok = torch.zeros(T, H, 2, dtype=torch.float32, device=gz.device)
+    floor = torch.zeros(T, H, dtype=torch.float32, device=gz.device)
+    cu = cu_q.tolist()
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        slot = int(state_slots[b])
+        m = torch.zeros(H, dtype=torch.float32, device=gz.device) if int(positions[q0]) == 0 \
+            else m_state[slot].clone()
+        for t in range(q0, q1):
+            m1 = torch.maximum(lf[t] + m, li[t])
+            tok[t, :, 0] = torch.exp(lf[t] + m - m1)
+            tok[t, :, 1] = torch.exp(li[t] - m1)
+            floor[t] = torch.exp(-m1)
+            m = m1
+        m_state[slot] = m
+    return tok, floor
+
+
+def matrix_memory_inputs(u, H: int, D: int, Dv: int):
+    """The recurrence inputs of a matrix memory from the projected rows u [T,
+    >= 2 H D + H Dv] (q | k | v): f32 [T, 2 H D + H (Dv + 1)] = q D^(-1/2) | k |
+    per head (v, 1) - the constant column makes the state's last column the
+    normaliser vector."""
+    T = u.shape[0]
+    q = u[:, :H * D].float() * D ** -0.5
+    k = u[:, H * D:2 * H * D].float()
+    v = u[:, 2 * H * D:2 * H * D + H * Dv].float().view(T, H, Dv)
+    v1 = torch.cat([v, torch.ones(T, H, 1, dtype=torch.float32, device=u.device)], dim=-1)
+    return torch.cat([q, k, v1.view(T, H * (Dv + 1))], dim=1).contiguous()
+
+
+def normalized_gated_rmsnorm(o, floor, w, gate, eps: float, out_dtype, H: int, Dv: int):
+    """o f32 [T, H (Dv + 1)]: per head Dv values and their normaliser dot; each
+    head's values are divided by max(|dot|, floor[t, h]) + 1e-6, then by their
+    root mean square over the head, times w [H Dv], times sigmoid(gate)."""
+    T = o.shape[0]
+    oh = o.float().view(T, H, Dv + 1)
+    y = oh[:, :, :Dv] / (torch.maximum(oh[:, :, Dv].abs(), floor.float()) + 1e-6)[:, :, None]
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+    return (y.reshape(T, H * Dv) * w.float() * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def delta_prep(u, gz, G: int, D: int, H: int, Dv: int, conv_w, tail, a_neg, dt_bias, state_slots,
+               cu_q, positions):
+    """The input stage of a gated delta rule over a flat token batch. u [T, >=
+    C], C = 2 G D + H Dv: the projected q | k | v rows pass a causal
+    convolution per channel (weights tap-major [taps, C], the last tap is the
+    current token's, no bias; rows before the feed from ``tail[slot]``, zeros
+    before position 0) and SiLU; every q and k head becomes a unit vector x /
+    sqrt(sum x^2 + 1e-6), q also times D^(-1/2) -> f32 [T, C]. gz f32 [T, 2 H]:
+    the first H columns give beta = sigmoid(z), the others the decay exp(a_neg
+    softplus(z + dt_bias)) -> f32 [T, H, 2] = (decay, beta)."""
+    T = u.shape[0]
+    taps, C = conv_w.shape
+    cu = cu_q.tolist()
+    xin = u[:, :C].float()
+    y = torch.zeros(T, C, dtype=torch.float32, device=u.device)
+    w = conv_w.float()
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        if taps > 1:
+            old = torch.zeros_like(tail[0]) if int(positions[q0]) == 0 else \
+                tail[int(state_slots[b])]
+            rows = torch.cat([old.float(), xin[q0:q1]])
+        else:
+            rows = xin[q0:q1]
+        n = q1 - q0
+        for j in range(taps):
+            y[q0:q1] += rows[j:j + n] * w[j]
+    y = torch.nn.functional.silu(y)
+    qk = y[:, :2 * G * D].view(T, 2 * G, D)
+    qk = qk * torch.rsqrt(qk.pow(2).sum(-1, keepdim=True) + 1e-6)
+    qk[:, :G] *= D ** -0.5
+    act = torch.cat([qk.reshape(T, 2 * G * D), y[:, 2 * G * D:]], dim=1).contiguous()
+    z = gz.float()
+    beta = torch.sigmoid(z[:, :H])
+    decay = torch.exp(a_neg.float() * torch.nn.functional.softplus(z[:, H:] + dt_bias.float()))
+    return act, torch.stack([decay, beta], dim=-1).contiguous()
+
+
+def delta_scan(act, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int, hpg: int, state,
+               state_slots, cu_q, positions, tok):
+    """The gated delta rule, token by token in f32, per sequence and head:
+
+        S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+
+    with (g, beta) = ``tok[t, h]``. ``act`` f32 [T, W]: head h reads q at
+    ``q_off + (h // hpg) D``, k at ``k_off + (h // hpg) D`` and v at ``v_off +
+    h Dv``. The state [slots, H, D, Dv] is read at the sequence's slot (zero
+    when the step's first position is 0) and written back. Returns o f32
+    [T, H Dv]."""
+    T = act.shape[0]
+    a = act.float()
+    hg = torch.arange(H, device=act.device) // hpg
+    cols = torch.arange(D, device=act.device)
+    q = a[:, (q_off + hg[:, None] * D + cols[None, :]).reshape(-1)].view(T, H, D)
+    k = a[:, (k_off + hg[:, None] * D + cols[None, :]).reshape(-1)].view(T, H, D)
+    v = a[:, v_off:v_off + H * Dv].view(T, H, Dv)
+    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=act.device)
+    cu = cu_q.tolist()
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        slot = int(state_slots[b])
+        S = torch.zeros_like(state[slot]) if int(positions[q0]) == 0 else state[slot].clone()
+        for t in range(q0, q1):
+            S = tok[t, :, 0].float()[:, None, None] * S
+            r = torch.einsum("hde,hd->he", S, k[t])
+            uu = tok[t, :, 1].float()[:, None] * (v[t] - r)
+            S = S + k[t][:, :, None] * uu[:, None, :]
+            o[t] = torch.einsum("hde,hd->he", S, q[t])
+        state[slot] = S
+    return o.view(T, H * Dv)

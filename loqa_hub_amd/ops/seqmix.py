@@ -308,14 +308,16 @@ def state_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: in
 
 
 def gated_rmsnorm(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, eps: float,
-                  out_dtype, groups: int = 1, silu_first: bool = False) -> torch.Tensor:
-    """y = rmsnorm(o) * w * sigmoid(gate) over whole rows of o f32 [T, n], or
-    with ``silu_first`` y = rmsnorm(o * silu(gate)) * w (the gate before the
-    norm); ``groups`` > 1 normalises a row in that many equal parts, each by
-    its own root mean square. ``gate`` [T, n] may be a column slice of a wider
-    projection."""
+                  out_dtype, groups: int = 1, silu_first: bool = False,
+                  gate_act: str = "sigmoid") -> torch.Tensor:
+    """y = rmsnorm(o) * w * sigmoid(gate) over whole rows of o f32 [T, n]
+    (``gate_act`` "silu": times silu(gate) instead), or with ``silu_first`` y =
+    rmsnorm(o * silu(gate)) * w (the gate before the norm); ``groups`` > 1
+    normalises a row in that many equal parts, each by its own root mean
+    square. ``gate`` [T, n] may be a column slice of a wider projection."""
+    assert gate_act in ("sigmoid", "silu")
     if not o.is_cuda:
-        return ref.gated_rmsnorm(o, w, gate, eps, out_dtype, groups, silu_first)
+        return ref.gated_rmsnorm(o, w, gate, eps, out_dtype, groups, silu_first, gate_act)
     _f32c(o, "o"); _f32c(w, "w")
     T, n = o.shape
     assert gate.shape == (T, n) and gate.stride(1) == 1 and w.numel() == n
@@ -323,7 +325,8 @@ def gated_rmsnorm(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, eps: flo
     y = torch.empty(T, n, dtype=out_dtype, device=o.device)
     if T:
         check(kernels().loqa_gated_rmsnorm(ptr(o), ptr(w), ptr(gate), _dt(gate), gate.stride(0), eps,
-                                           ptr(y), _dt(y), T, n, groups, int(silu_first),
+                                           ptr(y), _dt(y), T, n, groups,
+                                           1 if silu_first else (2 if gate_act == "silu" else 0),
                                            stream_ptr(o)), "gated_rmsnorm")
     return y
 
@@ -661,7 +664,8 @@ def scaled_add_rms1p(resid: torch.Tensor, y: torch.Tensor, ls: torch.Tensor,
 def qk_prep_append(u: torch.Tensor, H: int, G: int, D: int, Dv: int, v_off: int,
                    cos_sin: torch.Tensor | None, dims: int, eps: float, q_temp: tuple | None,
                    positions: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                   slots: torch.Tensor, out_dtype) -> torch.Tensor:
+                   slots: torch.Tensor, out_dtype, q_norm: torch.Tensor | None = None,
+                   k_norm: torch.Tensor | None = None) -> torch.Tensor:
     """One launch between the fused q | k (| v) projection u [T, W] and
     attention: per head the first ``dims`` entries of q and k rotate pairwise
     (interleaved layout, table ``cos_sin`` [positions, dims / 2, 2]), then q and
@@ -670,10 +674,17 @@ def qk_prep_append(u: torch.Tensor, H: int, G: int, D: int, Dv: int, v_off: int,
     + 1) (``q_temp`` = (coef, every) or None); k goes to its pages [blocks, BLK,
     G D] and the value rows - the columns at ``v_off``, or with ``v_off`` < 0
     the k columns as projected - to theirs [blocks, BLK, G Dv]. Returns q
-    [T, H D]. Statistics, angles and the temperature are f32."""
+    [T, H D]. Statistics, angles and the temperature are f32. With ``q_norm``
+    [H D] and ``k_norm`` [G D] (f32) the norm is another one: q and k are
+    RMS-normed over their whole projection with these weights BEFORE the
+    rotation, and no per-head division follows."""
+    assert (q_norm is None) == (k_norm is None)
     if not u.is_cuda:
         return ref.qk_prep_append(u, H, G, D, Dv, v_off, cos_sin, dims, eps, q_temp, positions,
-                                  k_cache, v_cache, slots, out_dtype)
+                                  k_cache, v_cache, slots, out_dtype, q_norm, k_norm)
+    if q_norm is not None:
+        _f32c(q_norm, "q_norm"); _f32c(k_norm, "k_norm")
+        assert q_norm.numel() == H * D and k_norm.numel() == G * D
     T, W = u.shape
     assert u.stride(1) == 1 and (H + G) * D <= W
     assert v_off < 0 and Dv == D or v_off >= (H + G) * D and v_off + G * Dv <= W
@@ -693,7 +704,7 @@ def qk_prep_append(u: torch.Tensor, H: int, G: int, D: int, Dv: int, v_off: int,
             ptr(u), _dt(u), u.stride(0), H, G, D, Dv, int(v_off), ptr(cos_sin) if dims else None,
             cos_sin.shape[0] if dims else 0, dims, float(eps), coef, every, ptr(positions),
             ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0], ptr(slots), ptr(q), T,
-            stream_ptr(u)), "qk_prep_append")
+            ptr(q_norm), ptr(k_norm), stream_ptr(u)), "qk_prep_append")
     return q
 
 
@@ -705,7 +716,8 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      positions: torch.Tensor, scale: float, softcap: float, window: int,
                      keep_first: int, gate: torch.Tensor | None, H: int, G: int, D: int, Dv: int,
                      max_q: int = 0, matrix_cores: bool | None = None, max_ctx: int = 0,
-                     key_splits: int | None = None) -> torch.Tensor:
+                     key_splits: int | None = None, sink: torch.Tensor | None = None
+                     ) -> torch.Tensor:
     """Softmax attention over paged K [blocks, BLK, G D] and V [blocks, BLK,
     G Dv] (query head h reads key/value head h // (H / G)): score = q . k *
     scale, soft-capped to cap tanh(score / cap) when ``softcap`` > 0; a query at
@@ -717,10 +729,15 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     batches are one launch. Scores, softmax and accumulators are f32. A step
     with few rows over long contexts (``max_ctx``) deals each row's keys out to
     ``key_splits`` workgroups (chosen here when None) and merges their partial
-    results in a second launch."""
+    results in a second launch. ``sink`` f32 [H]: head h's softmax denominator
+    also holds exp(sink[h]), a term that carries no value."""
     if not q.is_cuda:
         return ref.window_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions,
-                                    scale, softcap, window, keep_first, gate, H, G, D, Dv, q.dtype)
+                                    scale, softcap, window, keep_first, gate, H, G, D, Dv, q.dtype,
+                                    sink)
+    if sink is not None:
+        _f32c(sink, "sink")
+        assert sink.numel() == H
     T = q.shape[0]
     assert q.is_contiguous() and q.shape[1] == H * D and H % G == 0
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
@@ -756,8 +773,8 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             ptr(q), _dt(q), ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0],
             ptr(cu_q), ptr(ctx_lens), ptr(block_tables), block_tables.shape[1], ptr(positions),
             ptr(gate), gs, float(scale), float(softcap), int(window), int(keep_first), B, T, H, G,
-            D, Dv, int(max_q), int(mfma), ptr(o), int(key_splits), ptr(part), stream_ptr(q)),
-            "window_attention")
+            D, Dv, int(max_q), int(mfma), ptr(o), int(key_splits), ptr(part), ptr(sink),
+            stream_ptr(q)), "window_attention")
     return o
 
 
@@ -793,3 +810,221 @@ def mamba2_prep(u: torch.Tensor, x_off: int, C: int, dt_off: int, Hh: int, conv_
             ptr(dt_bias), ptr(a_neg), ptr(tail), tail.shape[0], ptr(state_slots), ptr(cu_q),
             ptr(positions), B, T, ptr(xbc), ptr(tok), stream_ptr(u)), "mamba2_prep")
     return xbc, tok
+
+
+# ---------------------------------------------------------------------------
+# Parallel layers (two norms of one residual, several sublayer outputs added
+# at once), the gate scan and input stage of a stabilised matrix memory, the
+# gated delta rule, and small steps around latent attention and the logits
+# (csrc/kernels/norm_rms1p.hip, matrix_memory.hip, delta_rule.hip)
+def residual_rms1p(resid: torch.Tensor, addends: list, extra: torch.Tensor | None,
+                   w_a: torch.Tensor | None, w_b: torch.Tensor | None, eps: float, out_dtype
+                   ) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+    """The residual step of a layer whose sublayers run side by side: resid
+    (f32, in place) += sum_i scale_i * y_i over up to three ``addends`` (tensor
+    [rows, d] in one activation dtype, scalar scale) and ``extra`` (f32 [rows,
+    d]); the same launch returns the two normed inputs of the next layer, h_a =
+    resid / rms(resid) * (1 + w_a) and h_b likewise with w_b (None where the
+    weight is None). Without addends it is the two norms alone."""
+    if not resid.is_cuda:
+        return ref.residual_rms1p(resid, addends, extra, w_a, w_b, eps, out_dtype)
+    _f32c(resid, "resid")
+    rows, d = resid.shape
+    assert len(addends) <= 3
+    ys = [None, None, None]
+    sc = [0.0, 0.0, 0.0]
+    ydt = 0
+    for i, (y, s_) in enumerate(addends):
+        assert y.shape == resid.shape and y.is_contiguous()
+        assert i == 0 or y.dtype == addends[0][0].dtype
+        ys[i], sc[i], ydt = y, float(s_), _dt(y)
+    if extra is not None:
+        _f32c(extra, "extra")
+        assert extra.shape == resid.shape
+    hs = []
+    for w in (w_a, w_b):
+        if w is None:
+            hs.append(None)
+            continue
+        _f32c(w, "norm weight")
+        assert w.numel() == d
+        hs.append(torch.empty(rows, d, dtype=out_dtype, device=resid.device))
+    if rows:
+        check(kernels().loqa_residual_rms1p(
+            ptr(resid), ptr(ys[0]), sc[0], ptr(ys[1]), sc[1], ptr(ys[2]), sc[2], ydt, ptr(extra),
+            ptr(w_a), ptr(w_b), float(eps), ptr(hs[0]), ptr(hs[1]), _DT[out_dtype], rows, d,
+            stream_ptr(resid)), "residual_rms1p")
+    return hs[0], hs[1]
+
+
+def rms_norm_cols(u: torch.Tensor, n: int, w: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """RMS norm with a plain weight over the first ``n`` columns of the rows of
+    u [T, >= n] (a slice of a fused projection) -> [T, n]; statistics f32."""
+    if not u.is_cuda:
+        return ref.rms_norm_cols(u, n, w, eps, out_dtype)
+    T = u.shape[0]
+    assert u.stride(1) == 1 and 0 < n <= u.shape[1]
+    _f32c(w, "w")
+    assert w.numel() == n
+    y = torch.empty(T, n, dtype=out_dtype, device=u.device)
+    if T:
+        check(kernels().loqa_rms_norm_cols(ptr(u), _dt(u), u.stride(0), n, ptr(w), float(eps),
+                                           ptr(y), _dt(y), T, stream_ptr(u)), "rms_norm_cols")
+    return y
+
+
+def sigmoid_gate_(o: torch.Tensor, gate: torch.Tensor, H: int, Dv: int) -> torch.Tensor:
+    """In place: the first Dv entries of every head of o [T, H, Dvo] (Dvo >= Dv:
+    heads may be padded) times sigmoid(gate [T, H Dv]); ``gate`` may be a
+    column slice of a wider projection."""
+    if not o.is_cuda:
+        return ref.sigmoid_gate_(o, gate, H, Dv)
+    T, Ho, Dvo = o.shape
+    assert Ho == H and Dvo >= Dv and o.is_contiguous()
+    assert gate.shape == (T, H * Dv) and gate.stride(1) == 1 and gate.dtype == o.dtype
+    if T:
+        check(kernels().loqa_sigmoid_gate(ptr(o), _dt(o), ptr(gate), gate.stride(0), T, H, Dvo, Dv,
+                                          stream_ptr(o)), "sigmoid_gate")
+    return o
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap tanh(x / cap) in place over a contiguous f32 tensor."""
+    if not x.is_cuda:
+        return ref.softcap_(x, cap)
+    _f32c(x, "x")
+    assert cap > 0
+    if x.numel():
+        check(kernels().loqa_softcap(ptr(x), x.numel(), float(cap), stream_ptr(x)), "softcap")
+    return x
+
+
+def exp_gate_scan(gz: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float,
+                  m_state: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+                  positions: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The gates of a stabilised exponential-gate memory over a flat token
+    batch. gz f32 [T, 2 H]: the pre-activations of the input gates (first H
+    columns) and the forget gates. Per head li = cap tanh((z_i + b_i) / cap),
+    lf = logsigmoid(cap tanh((z_f + b_f) / cap)) and the running maximum m_t =
+    max(lf + m_{t-1}, li), which is 0 before position 0 and otherwise carried
+    in ``m_state`` [slots, H] f32 (updated here). Returns tok f32 [T, H, 2] =
+    (exp(lf + m_{t-1} - m_t), exp(li - m_t)), the decay and the input scale of
+    the state recurrence, and floor f32 [T, H] = exp(-m_t)."""
+    if not gz.is_cuda:
+        return ref.exp_gate_scan(gz, i_bias, f_bias, cap, m_state, state_slots, cu_q, positions)
+    _f32c(gz, "gz"); _f32c(i_bias, "i_bias"); _f32c(f_bias, "f_bias"); _f32c(m_state, "m_state")
+    T, H2 = gz.shape
+    H = H2 // 2
+    assert H2 == 2 * H and i_bias.numel() == H and f_bias.numel() == H and cap > 0
+    assert m_state.shape[1:] == (H,)
+    B = _seq_args(state_slots, cu_q, positions, T)
+    tok = torch.empty(T, H, 2, dtype=torch.float32, device=gz.device)
+    floor = torch.empty(T, H, dtype=torch.float32, device=gz.device)
+    if T:
+        check(kernels().loqa_exp_gate_scan(ptr(gz), H, ptr(i_bias), ptr(f_bias), float(cap),
+                                           ptr(m_state), m_state.shape[0], ptr(state_slots),
+                                           ptr(cu_q), ptr(positions), B, T, ptr(tok), ptr(floor),
+                                           stream_ptr(gz)), "exp_gate_scan")
+    return tok, floor
+
+
+def matrix_memory_inputs(u: torch.Tensor, H: int, D: int, Dv: int) -> torch.Tensor:
+    """The recurrence inputs of a matrix memory from the projected rows u [T,
+    >= 2 H D + H Dv] (q | k | v): f32 [T, 2 H D + H (Dv + 1)] = q D^(-1/2) | k |
+    per head (v, 1). With the constant column, :func:`state_scan` over Dv + 1
+    value columns keeps the normaliser vector as the state's last column and
+    returns its product with q as every head's last output."""
+    if not u.is_cuda:
+        return ref.matrix_memory_inputs(u, H, D, Dv)
+    T = u.shape[0]
+    assert u.stride(1) == 1 and u.shape[1] >= 2 * H * D + H * Dv
+    act = torch.empty(T, 2 * H * D + H * (Dv + 1), dtype=torch.float32, device=u.device)
+    if T:
+        check(kernels().loqa_matrix_memory_inputs(ptr(u), _dt(u), u.stride(0), H, D, Dv, ptr(act),
+                                                  T, stream_ptr(u)), "matrix_memory_inputs")
+    return act
+
+
+def normalized_gated_rmsnorm(o: torch.Tensor, floor: torch.Tensor, w: torch.Tensor,
+                             gate: torch.Tensor, eps: float, out_dtype, H: int, Dv: int
+                             ) -> torch.Tensor:
+    """The output stage of a matrix memory. o f32 [T, H (Dv + 1)]: per head Dv
+    read-out values and the normaliser's product with q; each head's values are
+    divided by max(|product|, floor[t, h]) + 1e-6, then by their root mean
+    square over the head, times w [H Dv], times sigmoid(gate [T, H Dv]) (may be
+    a column slice). Returns [T, H Dv]."""
+    if not o.is_cuda:
+        return ref.normalized_gated_rmsnorm(o, floor, w, gate, eps, out_dtype, H, Dv)
+    _f32c(o, "o"); _f32c(floor, "floor"); _f32c(w, "w")
+    T = o.shape[0]
+    assert o.shape[1] == H * (Dv + 1) and floor.shape == (T, H) and w.numel() == H * Dv
+    assert gate.shape == (T, H * Dv) and gate.stride(1) == 1
+    y = torch.empty(T, H * Dv, dtype=out_dtype, device=o.device)
+    if T:
+        check(kernels().loqa_normalized_gated_rmsnorm(
+            ptr(o), ptr(floor), ptr(w), ptr(gate), _dt(gate), gate.stride(0), float(eps), ptr(y),
+            _dt(y), T, H, Dv, stream_ptr(o)), "normalized_gated_rmsnorm")
+    return y
+
+
+def delta_prep(u: torch.Tensor, gz: torch.Tensor, G: int, D: int, H: int, Dv: int,
+               conv_w: torch.Tensor, tail: torch.Tensor, a_neg: torch.Tensor,
+               dt_bias: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+               positions: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The input stage of a gated delta rule, one launch over a flat token
+    batch. The first C = 2 G D + H Dv columns of the projected rows u [T, W] (q
+    | k | v) pass a causal convolution per channel (f32 weights tap-major [taps,
+    C], last tap = the current token, no bias; the rows before a feed from
+    ``tail[slot]`` f32 [slots, taps - 1, C], zeros before position 0) and SiLU;
+    every q and k head becomes a unit vector x / sqrt(sum x^2 + 1e-6), q also
+    times D^(-1/2) -> f32 [T, C]. gz f32 [T, 2 H]: the first H columns give the
+    write strengths beta = sigmoid(z), the others the decays exp(a_neg
+    softplus(z + dt_bias)) -> f32 [T, H, 2] = (decay, beta). ``tail`` is not
+    written here (:func:`seq_state_save` does, after every reader)."""
+    if not u.is_cuda:
+        return ref.delta_prep(u, gz, G, D, H, Dv, conv_w, tail, a_neg, dt_bias, state_slots, cu_q,
+                              positions)
+    T, W = u.shape
+    taps, C = conv_w.shape
+    assert C == 2 * G * D + H * Dv and u.stride(1) == 1 and C <= W
+    for t, name, n in ((conv_w, "conv_w", None), (tail, "tail", None), (a_neg, "a_neg", H),
+                       (dt_bias, "dt_bias", H), (gz, "gz", T * 2 * H)):
+        _f32c(t, name)
+        assert n is None or t.numel() == n
+    assert tail.shape[1:] == (taps - 1, C)
+    B = _seq_args(state_slots, cu_q, positions, T)
+    act = torch.empty(T, C, dtype=torch.float32, device=u.device)
+    tok = torch.empty(T, H, 2, dtype=torch.float32, device=u.device)
+    if T:
+        check(kernels().loqa_delta_prep(
+            ptr(u), _dt(u), u.stride(0), ptr(gz), G, D, H, Dv, ptr(conv_w), taps, ptr(tail),
+            tail.shape[0], ptr(a_neg), ptr(dt_bias), ptr(state_slots), ptr(cu_q), ptr(positions), B,
+            T, ptr(act), ptr(tok), stream_ptr(u)), "delta_prep")
+    return act, tok
+
+
+def delta_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int,
+               hpg: int, state: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+               positions: torch.Tensor, tok: torch.Tensor) -> torch.Tensor:
+    """The gated delta rule with a carried matrix state, per sequence and head,
+    token by token in f32:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;
+    o = S^T q, with (g, beta) = ``tok[t, h]``. ``act`` f32 [T, W]: head h reads
+    q at ``q_off + (h // hpg) D``, k at ``k_off + (h // hpg) D`` and v at
+    ``v_off + h Dv``. ``state`` [slots, H, D, Dv] f32 carries S between steps
+    (zero when the step's first position is 0). One kernel and one order of
+    operations for prompt portions and single tokens."""
+    if not act.is_cuda:
+        return ref.delta_scan(act, H, D, Dv, q_off, k_off, v_off, hpg, state, state_slots, cu_q,
+                              positions, tok)
+    T, W = act.shape
+    _f32c(act, "act"); _f32c(state, "state"); _f32c(tok, "tok")
+    assert state.shape[1:] == (H, D, Dv) and hpg >= 1 and H % hpg == 0 and tok.shape == (T, H, 2)
+    G = H // hpg
+    assert min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + G * D <= W and v_off + H * Dv <= W
+    B = _seq_args(state_slots, cu_q, positions, T)
+    o = torch.empty(T, H * Dv, dtype=torch.float32, device=act.device)
+    if T:
+        check(kernels().loqa_delta_scan(ptr(act), W, H, D, Dv, q_off, k_off, v_off, hpg, ptr(state),
+                                        state.shape[0], ptr(state_slots), ptr(cu_q), ptr(positions),
+                                        ptr(tok), ptr(o), B, T, stream_ptr(act)), "delta_scan")
+    return o
