@@ -55,6 +55,7 @@ struct WinAttnParams {
   const void* gate; long gate_ld; float scale, cap; int window, keep_first;
   int B, T, H, G, D, Dv; void* o;
   int ns; float* part;               // key splits over workgroups and their partial results
+  const float* sink;                 // [H] or null: exp(sink[h]) joins head h's softmax denominator
 };
 
 // K / V pages (and the block table) are read through pointers in the global
@@ -121,12 +122,30 @@ __global__ __launch_bounds__(256) void qk_prep_append_kernel(
     const T* __restrict__ u, long ldu, int H, int G, int D, int Dv, int v_off,
     const float* __restrict__ cs, int max_pos, int dims, float eps, float coef, int every,
     const int* __restrict__ pos, T* __restrict__ kc, T* __restrict__ vc, long cache_rows,
-    const int* __restrict__ kvslots, T* __restrict__ q) {
+    const int* __restrict__ kvslots, T* __restrict__ q, const float* __restrict__ qn,
+    const float* __restrict__ kn) {
+  __shared__ float wsum[2][4];
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int p = pos[t];
   const long slot = kvslots[t];
   const bool store = slot >= 0 && slot < cache_rows;
   const T* ur = u + (size_t)t * ldu;
+  // the other norm: q and k RMS-normed over their whole projection, with
+  // weights, before the rotation (then no per-head division)
+  float invq = 1.f, invk = 1.f;
+  if (qn) {
+    float sq = 0.f, sk = 0.f;
+    for (int c = threadIdx.x; c < (H + G) * D; c += blockDim.x) {
+      const float v = Act<T>::ld(ur + c);
+      if (c < H * D) sq += v * v; else sk += v * v;
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) { wsum[0][wave] = sq; wsum[1][wave] = sk; }
+    __syncthreads();
+    invq = 1.f / sqrtf((wsum[0][0] + wsum[0][1] + wsum[0][2] + wsum[0][3]) / (float)(H * D) + eps);
+    invk = 1.f / sqrtf((wsum[1][0] + wsum[1][1] + wsum[1][2] + wsum[1][3]) / (float)(G * D) + eps);
+  }
   const float* csr = dims ? cs + (size_t)min(max(p, 0), max_pos - 1) * dims : nullptr;
   const float temp = 1.f + coef * logf((float)((p + 1) / every) + 1.f);
   constexpr int NP = 4;                           // pairs per lane (D <= 512)
@@ -147,6 +166,12 @@ __global__ __launch_bounds__(256) void qk_prep_append_kernel(
           Act<T>::st(vr, a[i]);
           Act<T>::st(vr + 1, b[i]);
         }
+        if (qn) {
+          const float* wn = isq ? qn + (size_t)job * D + e : kn + (size_t)(job - H) * D + e;
+          const float iv = isq ? invq : invk;
+          a[i] *= iv * wn[0];
+          b[i] *= iv * wn[1];
+        }
         if (e < dims) {
           const float c = csr[e], s = csr[e + 1];
           const float x = a[i] * c - b[i] * s, y = b[i] * c + a[i] * s;
@@ -157,7 +182,7 @@ __global__ __launch_bounds__(256) void qk_prep_append_kernel(
       }
     }
     ss = wave_sum(ss);
-    float inv = 1.f / sqrtf(ss / (float)D + eps);
+    float inv = qn ? 1.f : 1.f / sqrtf(ss / (float)D + eps);
     if (isq) inv *= temp;
     T* dst = isq ? q + (size_t)t * H * D + (size_t)job * D
                  : (store ? kc + (size_t)slot * G * D + (size_t)(job - H) * D : nullptr);
@@ -375,10 +400,12 @@ __global__ __launch_bounds__(64 * NW) void window_attn_keys_kernel(WinAttnParams
   __syncthreads();
   for (int idx = threadIdx.x; idx < nr * Dv; idx += blockDim.x) {
     const int r = idx / Dv, e = idx - r * Dv;
-    float M = -INFINITY;
+    const int h = g * rep + r0 + r;
+    const bool snk = p.sink && p.ns == 1;            // with key splits the combine launch adds it
+    float M = snk ? p.sink[h] : -INFINITY;
 #pragma unroll
     for (int w = 0; w < NW; ++w) M = fmaxf(M, mm[w * REP + r]);
-    float num = 0.f, den = 0.f;
+    float num = 0.f, den = snk ? expf(p.sink[h] - M) : 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
       const float mw = mm[w * REP + r];
@@ -386,7 +413,6 @@ __global__ __launch_bounds__(64 * NW) void window_attn_keys_kernel(WinAttnParams
       num += f * aa[(size_t)(w * REP + r) * Dv + e];
       den += f * ll[w * REP + r];
     }
-    const int h = g * rep + r0 + r;
     if (p.ns > 1) {                                  // the combine launch finishes the row
       float* pr = p.part + (((size_t)t * p.H + h) * p.ns + sp) * (Dv + 2);
       if (e == 0) { pr[0] = M; pr[1] = den; }
@@ -406,10 +432,10 @@ template <typename T>
 __global__ __launch_bounds__(128) void window_attn_combine_kernel(WinAttnParams p) {
   const int t = blockIdx.x, h = blockIdx.y, Dv = p.Dv;
   const float* pr = p.part + ((size_t)t * p.H + h) * p.ns * (Dv + 2);
-  float M = -INFINITY;
+  float M = p.sink ? p.sink[h] : -INFINITY;
   for (int s = 0; s < p.ns; ++s) M = fmaxf(M, pr[(size_t)s * (Dv + 2)]);
   for (int e = threadIdx.x; e < Dv; e += blockDim.x) {
-    float num = 0.f, den = 0.f;
+    float num = 0.f, den = p.sink ? expf(p.sink[h] - M) : 0.f;
     for (int s = 0; s < p.ns; ++s) {
       const float* ps = pr + (size_t)s * (Dv + 2);
       const float f = ps[0] == -INFINITY ? 0.f : expf(ps[0] - M);
@@ -640,7 +666,14 @@ __global__ __launch_bounds__(64 * WM_WAVES) void window_attn_mfma_kernel(WinAttn
     }
   }
   if (!valid) return;
-  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  if (p.sink) {
+    // the running maximum and sum are in the base-2 domain
+    const float sl = p.sink[head] * 1.44269504088896f;
+    const float mx2 = fmaxf(m_run, sl);
+    const float a = __builtin_amdgcn_exp2f(m_run - mx2);
+    inv = a / (l_run * a + __builtin_amdgcn_exp2f(sl - mx2));
+  }
   bf16_t* orow = (bf16_t*)p.o + ((size_t)(q0 + qi) * p.H + head) * DV;
   const bf16_t* grow = p.gate ? (const bf16_t*)p.gate + (size_t)(q0 + qi) * p.gate_ld + (size_t)head * DV
                               : nullptr;
@@ -694,16 +727,17 @@ extern "C" int loqa_qk_prep_append(const void* u, int dt, long ldu, int H, int G
                                    int v_off, const void* cs, int max_pos, int dims, float eps,
                                    float coef, int every, const void* pos, void* kc, void* vc,
                                    int blk, int nblocks, const void* kvslots, void* q, int T,
-                                   hipStream_t st) {
+                                   const void* qn, const void* kn, hipStream_t st) {
   if (T <= 0) return 0;
   if (D <= 0 || D > 512 || D % 2 || dims < 0 || dims > D || dims % 2 || every < 1 ||
-      (dims > 0 && (!cs || max_pos <= 0)) || H <= 0 || G <= 0)
+      (dims > 0 && (!cs || max_pos <= 0)) || H <= 0 || G <= 0 || (!qn) != (!kn))
     return (int)hipErrorInvalidValue;
   const long rows = (long)blk * nblocks;
 #define GO(TT)                                                                                  \
   hipLaunchKernelGGL(qk_prep_append_kernel<TT>, dim3(T), dim3(256), 0, st, (const TT*)u, ldu, H, \
                      G, D, Dv, v_off, (const float*)cs, max_pos, dims, eps, coef, every,        \
-                     (const int*)pos, (TT*)kc, (TT*)vc, rows, (const int*)kvslots, (TT*)q)
+                     (const int*)pos, (TT*)kc, (TT*)vc, rows, (const int*)kvslots, (TT*)q,      \
+                     (const float*)qn, (const float*)kn)
   if (dt == 0) GO(bf16_t); else GO(float);
 #undef GO
   return (int)hipGetLastError();
@@ -714,7 +748,8 @@ extern "C" int loqa_window_attention(const void* q, int dt, const void* kc, cons
                                      int max_blocks, const void* pos, const void* gate, long gate_ld,
                                      float scale, float cap, int window, int keep_first, int B,
                                      int T, int H, int G, int D, int Dv, int max_q, int mfma,
-                                     void* o, int ns, void* part, hipStream_t st) {
+                                     void* o, int ns, void* part, const void* sink,
+                                     hipStream_t st) {
   if (T <= 0) return 0;
   if (B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > 512 || Dv <= 0 || Dv > 512 || blk <= 0)
     return (int)hipErrorInvalidValue;
@@ -724,7 +759,7 @@ extern "C" int loqa_window_attention(const void* q, int dt, const void* kc, cons
   p.max_blocks = max_blocks; p.pos = (const int*)pos; p.gate = gate; p.gate_ld = gate_ld;
   p.scale = scale; p.cap = cap; p.window = window; p.keep_first = keep_first;
   p.B = B; p.T = T; p.H = H; p.G = G; p.D = D; p.Dv = Dv; p.o = o;
-  p.ns = 1; p.part = nullptr;
+  p.ns = 1; p.part = nullptr; p.sink = (const float*)sink;
   // the matrix-core form reads the gate in 8-byte runs
   const bool gate_ok = !gate || (gate_ld % 4 == 0 && ((size_t)gate & 7) == 0);
   if (mfma && dt == 0 && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) && gate_ok)

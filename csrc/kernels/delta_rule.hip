@@ -1,0 +1,276 @@
+// The gated delta rule over a flat token batch. Per sequence and head, with a
+// decay g_t and a write strength beta_t per token:
+//
+//   S <- g_t S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
+//
+// delta_prep_kernel: the input stage, one workgroup per token. The q | k | v
+// columns of the projected row pass a causal convolution per channel (weights
+// tap-major, the last tap is the current token's, no bias; rows before the feed
+// from the sequence's tail slot, zeros before position 0, so a reused slot
+// needs no clearing) and SiLU; q and k heads are staged in LDS, a wave per head
+// makes each a unit vector x / sqrt(sum x^2 + 1e-6) (q also times D^(-1/2)).
+// The gate rows give beta = sigmoid(z) and g = exp(a_neg softplus(z + dt_bias)).
+// Everything it writes is f32.
+//
+// delta_scan_kernel: one workgroup per (sequence, head, EC value columns). A
+// column of S never meets another column: u_e depends on column e of S only.
+// Sixteen neighbouring lanes share a column, each holding a contiguous run of
+// MAXD of its D rows in registers, so that the two products with the OLD
+// state that a token needs, S^T k and S^T q, are MAXD multiply-adds per lane
+// and one 16-lane sum each through data-parallel moves (no LDS, no barrier):
+//
+//   r = S^T k,  s = S^T q,  c = k . q        (before this token's update)
+//   u = beta (v - g r),   o = g s + u c,   S <- g S + k u
+//
+// which is the definition with the read-out folded in (S_new^T q = g S^T q + u
+// k . q). The state is stored with a column's rows side by side ([slots, H, Dv,
+// D]), so a wave reads and writes 4 D contiguous floats. The step's tokens are
+// staged TC at a time in LDS (rows zero-padded to 16 MAXD), the next group's
+// values already in flight in registers. The recurrence runs token by token
+// in f32; a prompt portion, a single token or any cut of a prompt is the same
+// sequence of operations, for any EC.
+#include "seqmix.h"
+#include <type_traits>
+
+#define DR_DP 16        // lanes per state column
+
+__device__ __forceinline__ int dr_seq_of_row(const int* __restrict__ cu_q, int B, int t) {
+  const int lane = threadIdx.x & 63;
+  int b = 0;
+  for (int base = 1; base < B; base += 64) {
+    const int i = base + lane;
+    const bool at_or_before = i < B && cu_q[i] <= t;
+    b += __popcll(__ballot(at_or_before));
+  }
+  return b;
+}
+
+__device__ __forceinline__ float dr_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+template <int CTRL> __device__ __forceinline__ float dr_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// the sum over each run of 16 lanes, in every lane of the run
+__device__ __forceinline__ float dr_sum16(float v) {
+  v += dr_dpp<0xB1>(v);              // lanes 1 0 3 2 of each four
+  v += dr_dpp<0x4E>(v);              // lanes 2 3 0 1 of each four
+  v += dr_dpp<0x141>(v);             // the other four of each eight (mirror)
+  v += dr_dpp<0x140>(v);             // the other eight of each sixteen (mirror)
+  return v;
+}
+
+template <typename TU>
+__global__ __launch_bounds__(256) void delta_prep_kernel(
+    const TU* __restrict__ u, long ldu, const float* __restrict__ gz, int G, int D, int H, int Dv,
+    const float* __restrict__ cw, int taps, const float* __restrict__ tail, int nslots,
+    const float* __restrict__ a_neg, const float* __restrict__ dt_bias,
+    const int* __restrict__ sslots, const int* __restrict__ cu_q, const int* __restrict__ pos,
+    int B, float* __restrict__ act, float* __restrict__ tok) {
+  extern __shared__ float qk[];                 // [2 G D] convolved q | k before the unit norm
+  const int t = blockIdx.x;
+  if (t >= cu_q[B]) return;
+  const int b = dr_seq_of_row(cu_q, B, t);
+  const int i = t - cu_q[b], p = pos[t], keep = taps - 1;
+  const int QK = 2 * G * D, C = QK + H * Dv;
+  const float* ts = tail + (size_t)min(max(sslots[b], 0), nslots - 1) * keep * C;
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    const float* z = gz + (size_t)t * 2 * H;
+    tok[((size_t)t * H + h) * 2] = expf(a_neg[h] * dr_softplus(z[H + h] + dt_bias[h]));
+    tok[((size_t)t * H + h) * 2 + 1] = sigmoid_f(z[h]);
+  }
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int s = keep - j;                   // how many tokens back this tap reads
+      if (p - s < 0) continue;                  // before the sequence's start
+      const float uv = i - s >= 0 ? Act<TU>::ld(u + (size_t)(t - s) * ldu + c)
+                                  : ts[(size_t)(keep + i - s) * C + c];
+      acc += cw[(size_t)j * C + c] * uv;
+    }
+    const float y = silu_f(acc);
+    if (c < QK) qk[c] = y; else act[(size_t)t * C + c] = y;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const float qscale = 1.f / sqrtf((float)D);
+  for (int hd = wid; hd < 2 * G; hd += nw) {
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) ss += qk[hd * D + d] * qk[hd * D + d];
+    ss = wave_sum(ss);
+    const float inv = (hd < G ? qscale : 1.f) / sqrtf(ss + 1e-6f);
+    for (int d = lane; d < D; d += 64) act[(size_t)t * C + hd * D + d] = qk[hd * D + d] * inv;
+  }
+}
+
+template <int MAXD, int TC, int EC>   // D <= DR_DP * MAXD
+__global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
+    const float* __restrict__ act, long ld, int H, int D, int Dv, int q_off, int k_off, int v_off,
+    int hpg, float* __restrict__ state, const int* __restrict__ state_slots,
+    const int* __restrict__ cu_q, const int* __restrict__ positions, const float* __restrict__ tok,
+    float* __restrict__ o) {
+  constexpr int NTH = EC * DR_DP;
+  constexpr int DPAD = DR_DP * MAXD;            // padded row length in LDS
+  constexpr int NPT = TC * DPAD / NTH;          // staged q (and k) values per thread
+  constexpr int NVT = (TC * EC + NTH - 1) / NTH;
+  __shared__ __attribute__((aligned(16))) float qs[TC * DPAD];
+  __shared__ __attribute__((aligned(16))) float ks[TC * DPAD];
+  __shared__ float vs[TC * EC];
+  __shared__ float os[TC * EC];
+  __shared__ float gs[TC], bs[TC];
+  const int b = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * EC;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (q1 <= q0) return;
+  const int tid = threadIdx.x;
+  const int dp = tid % DR_DP, e = tid / DR_DP;
+  const bool col = e0 + e < Dv;
+  // a column's rows side by side: state [slots, H, Dv, D]
+  float* Sg = state + (((size_t)state_slots[b] * H + h) * Dv + e0 + e) * D + dp * MAXD;
+  const bool fresh = positions[q0] == 0;
+  float S[MAXD];
+  if (!fresh && col && D % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < MAXD / 4; ++i) {
+      float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (dp * MAXD + 4 * i < D) s4 = *reinterpret_cast<const float4*>(Sg + 4 * i);
+      S[4 * i] = s4.x; S[4 * i + 1] = s4.y; S[4 * i + 2] = s4.z; S[4 * i + 3] = s4.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i)
+      S[i] = (!fresh && col && dp * MAXD + i < D) ? Sg[i] : 0.f;
+  }
+  const size_t qoff = (size_t)q_off + (size_t)(h / hpg) * D;
+  const size_t koff = (size_t)k_off + (size_t)(h / hpg) * D;
+  const size_t voff = (size_t)v_off + (size_t)h * Dv + e0;
+  float rq[NPT], rk[NPT], rv[NVT], rg = 1.f, rb = 0.f;
+  auto fetch = [&](int t0) {               // the values of tokens t0 .. t0 + TC into registers
+    if (tid < TC) {
+      const bool ok = t0 + tid < q1;
+      rg = ok ? tok[((size_t)(t0 + tid) * H + h) * 2] : 1.f;
+      rb = ok ? tok[((size_t)(t0 + tid) * H + h) * 2 + 1] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+      const int i = tid + NTH * j, tt = i / DPAD, d = i % DPAD;
+      const bool ok = t0 + tt < q1 && d < D;
+      const float* row = act + (size_t)(ok ? t0 + tt : q0) * ld;
+      rq[j] = ok ? row[qoff + d] : 0.f;
+      rk[j] = ok ? row[koff + d] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NVT; ++j) {
+      const int i = tid + NTH * j, tt = i / EC, c = i % EC;
+      const bool ok = i < TC * EC && t0 + tt < q1 && e0 + c < Dv;
+      rv[j] = ok ? act[(size_t)(t0 + tt) * ld + voff + c] : 0.f;
+    }
+  };
+  fetch(q0);
+  for (int t0 = q0; t0 < q1; t0 += TC) {
+    const int nt = min(TC, q1 - t0);
+    __syncthreads();                       // the previous group's LDS is consumed
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+      qs[tid + NTH * j] = rq[j];
+      ks[tid + NTH * j] = rk[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NVT; ++j)
+      if (tid + NTH * j < TC * EC) vs[tid + NTH * j] = rv[j];
+    if (tid < TC) { gs[tid] = rg; bs[tid] = rb; }
+    __syncthreads();
+    if (t0 + TC < q1) fetch(t0 + TC);      // in flight while this group is computed
+    for (int tt = 0; tt < nt; ++tt) {
+      float4 kc[MAXD / 4], qc[MAXD / 4];
+      const float4* k4 = reinterpret_cast<const float4*>(ks + tt * DPAD + dp * MAXD);
+      const float4* q4 = reinterpret_cast<const float4*>(qs + tt * DPAD + dp * MAXD);
+#pragma unroll
+      for (int i = 0; i < MAXD / 4; ++i) { kc[i] = k4[i]; qc[i] = q4[i]; }
+      float r0 = 0.f, r1 = 0.f, s0 = 0.f, s1 = 0.f, c0 = 0.f, c1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < MAXD / 4; ++i) {
+        r0 += S[4 * i] * kc[i].x;     s0 += S[4 * i] * qc[i].x;     c0 += kc[i].x * qc[i].x;
+        r1 += S[4 * i + 1] * kc[i].y; s1 += S[4 * i + 1] * qc[i].y; c1 += kc[i].y * qc[i].y;
+        r0 += S[4 * i + 2] * kc[i].z; s0 += S[4 * i + 2] * qc[i].z; c0 += kc[i].z * qc[i].z;
+        r1 += S[4 * i + 3] * kc[i].w; s1 += S[4 * i + 3] * qc[i].w; c1 += kc[i].w * qc[i].w;
+      }
+      const float r = dr_sum16(r0 + r1), sq = dr_sum16(s0 + s1), kq = dr_sum16(c0 + c1);
+      const float g = gs[tt];
+      const float uu = bs[tt] * (vs[tt * EC + e] - g * r);
+#pragma unroll
+      for (int i = 0; i < MAXD / 4; ++i) {
+        S[4 * i] = g * S[4 * i] + kc[i].x * uu;
+        S[4 * i + 1] = g * S[4 * i + 1] + kc[i].y * uu;
+        S[4 * i + 2] = g * S[4 * i + 2] + kc[i].z * uu;
+        S[4 * i + 3] = g * S[4 * i + 3] + kc[i].w * uu;
+      }
+      if (dp == 0) os[tt * EC + e] = g * sq + uu * kq;
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * EC; i += NTH) {
+      const int tt = i / EC, c = i % EC;
+      if (e0 + c < Dv) o[(size_t)(t0 + tt) * H * Dv + (size_t)h * Dv + e0 + c] = os[i];
+    }
+  }
+  if (col && D % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < MAXD / 4; ++i)
+      if (dp * MAXD + 4 * i < D)
+        *reinterpret_cast<float4*>(Sg + 4 * i) =
+            make_float4(S[4 * i], S[4 * i + 1], S[4 * i + 2], S[4 * i + 3]);
+  } else if (col) {
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i)
+      if (dp * MAXD + i < D) Sg[i] = S[i];
+  }
+}
+
+extern "C" int loqa_delta_prep(const void* u, int u_dt, long ldu, const void* gz, int G, int D,
+                               int H, int Dv, const void* cw, int taps, const void* tail,
+                               int nslots, const void* a_neg, const void* dt_bias,
+                               const void* sslots, const void* cu_q, const void* pos, int B, int T,
+                               void* act, void* tok, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (B <= 0 || taps < 1 || nslots <= 0 || G <= 0 || D <= 0 || H <= 0 || Dv <= 0 ||
+      (size_t)2 * G * D * 4 > 64 * 1024)
+    return (int)hipErrorInvalidValue;
+#define GO(TU)                                                                                   \
+  hipLaunchKernelGGL(delta_prep_kernel<TU>, dim3(T), dim3(256), (size_t)2 * G * D * 4, st,       \
+                     (const TU*)u, ldu, (const float*)gz, G, D, H, Dv, (const float*)cw, taps,   \
+                     (const float*)tail, nslots, (const float*)a_neg, (const float*)dt_bias,     \
+                     (const int*)sslots, (const int*)cu_q, (const int*)pos, B, (float*)act,      \
+                     (float*)tok)
+  if (u_dt == 0) GO(bf16_t); else GO(float);
+#undef GO
+  return (int)hipGetLastError();
+}
+
+// act: f32 [T, ld]; head h reads q at q_off + (h / hpg) D, k at k_off + (h / hpg) D,
+// v at v_off + h Dv; tok [T, H, 2] = (decay, beta); state [slots, H, Dv, D].
+extern "C" int loqa_delta_scan(const void* act, long ld, int H, int D, int Dv, int q_off, int k_off,
+                               int v_off, int hpg, void* state, int nslots,
+                               const void* state_slots, const void* cu_q, const void* positions,
+                               const void* tok, void* o, int B, int T, hipStream_t st) {
+  if (T <= 0 || B <= 0) return 0;
+  if (D > DR_DP * 16 || D <= 0 || Dv <= 0 || hpg <= 0 || H % hpg || !tok)
+    return (int)hipErrorInvalidValue;
+  (void)nslots;
+  // column block: 16 when (sequences x heads x column blocks) fill the GPU,
+  // narrower for a lone prompt
+  const long wg16 = (long)B * H * ((Dv + 15) / 16);
+  const int ec = wg16 >= 256 ? 16 : (wg16 * 2 >= 256 ? 8 : 4);
+#define GO(MD, TCC, ECC)                                                                          \
+  hipLaunchKernelGGL((delta_scan_kernel<MD, TCC, ECC>), dim3(B, H, (Dv + ECC - 1) / ECC),         \
+                     dim3(ECC * DR_DP), 0, st, (const float*)act, ld, H, D, Dv, q_off, k_off,     \
+                     v_off, hpg, (float*)state, (const int*)state_slots, (const int*)cu_q,        \
+                     (const int*)positions, (const float*)tok, (float*)o)
+#define GOE(MD, TCC)                                                                              \
+  do {                                                                                            \
+    if (ec == 16) GO(MD, TCC, 16); else if (ec == 8) GO(MD, TCC, 8); else GO(MD, TCC, 4);         \
+  } while (0)
+  if (D <= 64) GOE(4, 16);
+  else if (D <= 128) GOE(8, 16);
+  else GOE(16, 8);
+#undef GOE
+#undef GO
+  return (int)hipGetLastError();
+}

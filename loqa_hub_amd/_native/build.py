@@ -86,7 +86,8 @@ def _build_lib(name: str, sources: list[str], headers: list[str], flags: list[st
 # (seconds) and not the whole kernel set (minutes).
 SEQMIX_SOURCES = ("norm_dyt.hip", "attn_latent.hip", "attn_latent_prefill.hip", "lightning.hip",
                   "moe.hip", "seq_rows.hip", "norm_scalar.hip", "attn_sigmoid.hip",
-                  "norm_rms1p.hip", "attn_window.hip", "mamba2.hip")
+                  "norm_rms1p.hip", "attn_window.hip", "mamba2.hip", "matrix_memory.hip",
+                  "delta_rule.hip")
 
 # hipcc may not form packed-f32 VALU instructions from scalar float code
 NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

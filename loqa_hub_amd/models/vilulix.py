@@ -343,7 +343,7 @@ class VilulixModel:
             else:
                 a, d = m.left, m.right
                 kv[r] = (a.kv_heads * a.dim, a.kv_heads * a.vdim)
-                state[r] = (d.heads, d.dim, d.vdim)
+                state[r] = (d.heads, d.vdim, d.dim)        # a column's rows side by side
                 if d.taps > 1:
                     rows[r] = {"tail": (d.taps - 1, d.conv_channels)}
         return {"latent": latent, "state": state, "kv_rows": kv, "rows": rows}

@@ -1264,9 +1264,9 @@ def delta_scan(act, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int,
 
     with (g, beta) = ``tok[t, h]``. ``act`` f32 [T, W]: head h reads q at
     ``q_off + (h // hpg) D``, k at ``k_off + (h // hpg) D`` and v at ``v_off +
-    h Dv``. The state [slots, H, D, Dv] is read at the sequence's slot (zero
-    when the step's first position is 0) and written back. Returns o f32
-    [T, H Dv]."""
+    h Dv``. The state is kept with a column's rows side by side, [slots, H, Dv,
+    D]; it is read at the sequence's slot (zero when the step's first position
+    is 0) and written back. Returns o f32 [T, H Dv]."""
     T = act.shape[0]
     a = act.float()
     hg = torch.arange(H, device=act.device) // hpg
@@ -1281,12 +1281,13 @@ def delta_scan(act, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int,
         if q1 == q0:
             continue
         slot = int(state_slots[b])
-        S = torch.zeros_like(state[slot]) if int(positions[q0]) == 0 else state[slot].clone()
+        S = torch.zeros(H, D, Dv, dtype=torch.float32, device=act.device) \
+            if int(positions[q0]) == 0 else state[slot].transpose(1, 2).clone()
         for t in range(q0, q1):
             S = tok[t, :, 0].float()[:, None, None] * S
             r = torch.einsum("hde,hd->he", S, k[t])
             uu = tok[t, :, 1].float()[:, None] * (v[t] - r)
             S = S + k[t][:, :, None] * uu[:, None, :]
             o[t] = torch.einsum("hde,hd->he", S, q[t])
-        state[slot] = S
+        state[slot] = S.transpose(1, 2)
     return o.view(T, H * Dv)

@@ -1010,15 +1010,16 @@ def delta_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: in
     token by token in f32:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;
     o = S^T q, with (g, beta) = ``tok[t, h]``. ``act`` f32 [T, W]: head h reads
     q at ``q_off + (h // hpg) D``, k at ``k_off + (h // hpg) D`` and v at
-    ``v_off + h Dv``. ``state`` [slots, H, D, Dv] f32 carries S between steps
-    (zero when the step's first position is 0). One kernel and one order of
-    operations for prompt portions and single tokens."""
+    ``v_off + h Dv``. ``state`` [slots, H, Dv, D] f32 (a column's rows side by
+    side) carries S between steps (zero when the step's first position is 0).
+    One kernel and one order of operations for prompt portions and single
+    tokens."""
     if not act.is_cuda:
         return ref.delta_scan(act, H, D, Dv, q_off, k_off, v_off, hpg, state, state_slots, cu_q,
                               positions, tok)
     T, W = act.shape
     _f32c(act, "act"); _f32c(state, "state"); _f32c(tok, "tok")
-    assert state.shape[1:] == (H, D, Dv) and hpg >= 1 and H % hpg == 0 and tok.shape == (T, H, 2)
+    assert state.shape[1:] == (H, Dv, D) and hpg >= 1 and H % hpg == 0 and tok.shape == (T, H, 2)
     G = H // hpg
     assert min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + G * D <= W and v_off + H * Dv <= W
     B = _seq_args(state_slots, cu_q, positions, T)

@@ -1,0 +1,783 @@
+"""The Vilulix family through the framework (registry, weights, engine step,
+hybrid cache, scheduler) against the plain float64 oracle in
+``vilulix_oracle.py``. Every test builds its own small configuration and
+seeded weights. The same tests run on the CPU (reference ops) and, marked
+``gpu``, on the HIP kernels.
+"""
+import json
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import vilulix_oracle as O
+from loqa_hub_amd.engine.llm_engine import GenRequest, LLMEngine
+from loqa_hub_amd.models.configs import vilulix_config_from_json
+from loqa_hub_amd.models.registry import family_of, lm_config_from_json
+from loqa_hub_amd.models.vilulix import VilulixWeights, config_to_json, random_state_dict
+from loqa_hub_amd.ops import seqmix
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+TOL = {torch.float32: 2e-4, torch.bfloat16: 6e-2}
+F64 = torch.float64
+
+
+def engine(cfg_json, sd, device, dtype=torch.float32, max_tokens=256, block=16, max_seqs=4):
+    cfg = lm_config_from_json(cfg_json, "t")
+    w = VilulixWeights(cfg, sd, device, dtype, max_positions=max_tokens)
+    return LLMEngine(cfg, device, weights=w, max_seqs=max_seqs, max_seq_len=max_tokens,
+                     block_size=block, num_blocks=max_tokens // block, use_graphs=False, dtype=dtype)
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor, q: float = 1.0) -> float:
+    """RMS difference (mean removed per row) over the RMS of the wanted logits:
+    the worst row, or the ``q`` quantile of the rows."""
+    d = got.double().cpu() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want - want.mean(-1, keepdim=True)
+    return float((d.pow(2).mean(-1).sqrt() / w.pow(2).mean().sqrt()).quantile(q))
+
+
+def feed(eng, seq, toks, cuts):
+    """Feed ``toks`` to one sequence in portions of ``cuts`` sizes (cycled);
+    returns the logits of every position."""
+    out, i, k = [], 0, 0
+    while i < len(toks):
+        n = min(cuts[k % len(cuts)], len(toks) - i)
+        out.append(eng.step_logits([seq], [toks[i:i + n]], [list(range(n))]))
+        i, k = i + n, k + 1
+    return torch.cat(out)
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+# every mixer kind, a repeated stretch that holds all of them (so every pass
+# needs pages, states, maxima and tails of its own), grouped and ungrouped
+# heads, a layer without a feed-forward, partial and full rotation
+FULL = [(O.mlstm(), O.dense_ff()),
+        (O.latent(), O.dense_ff(24)),
+        (O.parallel(), O.dense_ff()),
+        (O.mlstm(heads=2, dim=12, vdim=6, cap=3.0), None),
+        (O.parallel(O.window_attn(heads=2, kv_heads=2, dim=8, vdim=8, window=20, dims=8),
+                    O.delta(heads=2, kv_heads=2, dim=6, vdim=10, conv=2), 1.0, 1.0), O.dense_ff(16))]
+
+
+@pytest.fixture(scope="module")
+def full_model():
+    cfg = O.make_config(FULL, loop=(0, 3, 2))
+    return cfg, O.make_weights(cfg, 1)
+
+
+def test_registry_reads_config(full_model):
+    cfg_json, _ = full_model
+    cfg = lm_config_from_json(json.loads(json.dumps(cfg_json)))
+    assert family_of(cfg).name == "vilulix" and family_of(cfg_json).hybrid
+    assert cfg.n_layers == len(FULL) and cfg.layers[3].mlp is None
+    assert cfg.layers[2].mixer.left.window == 6 and cfg.layers[2].mixer.left.zero_sink
+    assert cfg.layers[2].mixer.left.qk_norm == "whole" and cfg.layers[2].mixer.left.rot.half
+    assert cfg.layers[2].mixer.right.taps == 3 and cfg.layers[2].mixer.right_scale == 1.3
+    assert cfg.layers[1].mixer.q_rank == 14 and cfg.layers[1].mixer.gate
+    assert cfg.layers[0].mixer.gate_cap == 8.0 and cfg.logit_softcap == 10.0
+    assert [i for i, _ in cfg.runs()] == [0, 1, 2, 0, 1, 2, 3, 4]
+    assert [f for _, f in cfg.runs()] == [False, False, False, True, False, False, False, False]
+    assert config_to_json(cfg)["layers"] == json.loads(json.dumps(cfg_json))["layers"]
+    assert config_to_json(cfg)["loop"] == cfg_json["loop"]
+    for li, path, val in ((2, ("left", "kv_heads"), 3), (2, ("right", "kv_heads"), 3),
+                          (1, ("rot", "dims"), 6), (0, ("gate_cap",), 0.0)):
+        bad = json.loads(json.dumps(cfg_json))
+        m = bad["layers"][li]["mixer"]
+        for k in path[:-1]:
+            m = m[k]
+        m[path[-1]] = val
+        with pytest.raises(ValueError):
+            vilulix_config_from_json(bad)
+    bad = json.loads(json.dumps(cfg_json))
+    bad["loop"]["stop"] = 9
+    with pytest.raises(ValueError):
+        vilulix_config_from_json(bad)
+    sd = random_state_dict(cfg, 0)
+    assert sd["l2.mix.right.v.conv"].shape == (24, 3) and sd["l1.mix.dkv"].shape == (16, 32)
+    assert sd["l0.mix.i.b"].shape == (3,) and "l3.norm2" not in sd
+
+
+# ------------------------------------------------------ each mechanism alone
+def _meta(lens, starts, device):
+    cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+    pos = torch.cat([s + torch.arange(n) for n, s in zip(lens, starts)]).to(torch.int32)
+    return cu.to(device), pos.to(device)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("d", [40, 256, 4100])
+def test_two_norm_residual_step(device, d):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(9, d, generator=g)
+    ys = [torch.randn(9, d, generator=g) for _ in range(3)]
+    x0 = torch.randn(9, d, generator=g)
+    w1, w2 = (torch.randn(d, generator=g) * 0.3 for _ in range(2))
+    eps = 1e-3
+    ha, hb = seqmix.residual_rms1p(x.to(device).clone(), [], None, w1.to(device), None, eps,
+                                   torch.float32)
+    assert hb is None
+    assert (ha.cpu().double() - O.norm_around_zero(x.double(), w1.double(), eps)).abs().max() < 1e-5
+    for ydt in (torch.float32, torch.bfloat16):
+        for n, extra in ((1, False), (2, True), (3, True), (0, True)):
+            r = x.to(device).clone()
+            adds = [(ys[i].to(ydt).to(device), s) for i, s in zip(range(n), (1.0, 0.7, -1.3))]
+            ha, hb = seqmix.residual_rms1p(r, adds, x0.to(device) if extra else None,
+                                           w1.to(device), w2.to(device), eps, torch.float32)
+            want = x.double() + sum(s * y.double().cpu() for y, s in adds) + \
+                (x0.double() if extra else 0.0)
+            assert (r.cpu().double() - want).abs().max() < 1e-5
+            assert (ha.cpu().double() - O.norm_around_zero(want, w1.double(), eps)).abs().max() < 1e-5
+            assert (hb.cpu().double() - O.norm_around_zero(want, w2.double(), eps)).abs().max() < 1e-5
+    r = x.to(device).clone()
+    assert seqmix.residual_rms1p(r, [(ys[0].to(device), 2.0)], None, None, None, eps,
+                                 torch.float32) == (None, None)
+    assert (r.cpu().double() - (x.double() + 2.0 * ys[0].double())).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_small_steps(device):
+    """Plain-weight norm over a column slice, the output gate on padded heads,
+    the soft cap."""
+    g = torch.Generator().manual_seed(1)
+    u = torch.randn(7, 50, generator=g)
+    w = torch.randn(19, generator=g)
+    got = seqmix.rms_norm_cols(u.to(device), 19, w.to(device), 1e-4, torch.float32)
+    assert (got.cpu().double() - O.norm_plain(u[:, :19].double(), w.double(), 1e-4)).abs().max() < 1e-5
+    o = torch.randn(7, 3, 8, generator=g)
+    gt = torch.randn(7, 40, generator=g)
+    got = seqmix.sigmoid_gate_(o.to(device).clone(), gt.to(device)[:, 4:4 + 15], 3, 5)
+    want = o.double().clone()
+    want[:, :, :5] *= torch.sigmoid(gt[:, 4:19].double()).view(7, 3, 5)
+    assert (got.cpu().double() - want).abs().max() < 1e-6
+    z = torch.randn(5, 33, generator=g) * 20
+    got = seqmix.softcap_(z.to(device).clone(), 7.0)
+    assert (got.cpu().double() - 7.0 * torch.tanh(z.double() / 7.0)).abs().max() < 1e-5
+
+
+def _matrix_memory_case(device, m, cuts, dtype=torch.float32, seed=3, lens=(37, 1, 9), big=False):
+    """The mLSTM mixer's ops in the model's order, several sequences fed in
+    portions, against the oracle's mixer on the whole sequences."""
+    H, D, Dv, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
+    d = 24
+    g = torch.Generator().manual_seed(seed)
+    cfg = O.make_config([(("mlstm", m), None)], width=d)
+    sd = O.make_weights(cfg, seed)
+    if big:          # strong gates: the running maximum moves and the floor matters
+        sd["l0.mix.i"] *= 6.0
+        sd["l0.mix.f"] *= 6.0
+        sd["l0.mix.q"] *= 0.05
+    hs = [torch.randn(n, d, generator=g).to(dtype).float() for n in lens]
+    want = [O.mixer_mlstm({k: v.double() for k, v in sd.items()}, "l0.", m, h.double(), 1e-5)
+            for h in hs]
+    dev = torch.device(device)
+    p = "l0.mix."
+    w_in = torch.cat([sd[p + n] for n in "qkvg"]).to(dev, dtype)
+    w_g = torch.cat([sd[p + "i"], sd[p + "f"]]).to(dev)
+    state = torch.full((len(lens) + 1, H, D, Dv + 1), 9.0, device=dev)
+    mst = torch.full((len(lens) + 1, H), -3.0, device=dev)
+    slots = torch.tensor([2, 0, 1][:len(lens)], dtype=torch.int32, device=dev)
+    at = [0] * len(lens)
+    got = [[] for _ in lens]
+    k = 0
+    while any(a < n for a, n in zip(at, lens)):
+        feeds = [min(cuts[(k + b) % len(cuts)], n - a) for b, (a, n) in enumerate(zip(at, lens))]
+        cu, pos = _meta(feeds, at, dev)
+        h = torch.cat([hs[b][a:a + f] for b, (a, f) in enumerate(zip(at, feeds))]).to(dev, dtype)
+        u = torch.nn.functional.linear(h, w_in)
+        gz = torch.nn.functional.linear(h.float(), w_g)
+        tok, floor = seqmix.exp_gate_scan(gz, sd[p + "i.b"].to(dev), sd[p + "f.b"].to(dev), cap, mst,
+                                          slots, cu, pos)
+        act = seqmix.matrix_memory_inputs(u, H, D, Dv)
+        o = seqmix.state_scan(act, H, D, Dv + 1, 0, H * D, 2 * H * D, 1, state, slots, cu, pos,
+                              tok=tok)
+        y = seqmix.normalized_gated_rmsnorm(o, floor, sd[p + "norm"].to(dev),
+                                            u[:, 2 * H * D + H * Dv:], 1e-5, torch.float32, H, Dv)
+        y = y.cpu().double() @ sd[p + "o"].double().T
+        o0 = 0
+        for b, f in enumerate(feeds):
+            got[b].append(y[o0:o0 + f])
+            o0 += f
+            at[b] += f
+        k += 1
+    return [torch.cat(x) for x in got], want
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[37], [1], [2, 1, 3, 17, 1, 13]], ids=lambda c: str(len(c)))
+@pytest.mark.parametrize("m", [O.mlstm()[1], O.mlstm(1, 5, 3, 2.0)[1], O.mlstm(2, 64, 128, 12.0)[1],
+                               O.mlstm(2, 72, 31, 6.0)[1]], ids=lambda m: f"{m['dim']}x{m['vdim']}")
+def test_matrix_memory_mixer(device, m, cuts):
+    for big in (False, True):
+        got, want = _matrix_memory_case(device, m, cuts, big=big)
+        for a, b in zip(got, want):
+            assert (a - b).abs().max() < 3e-4 * max(1.0, float(b.abs().max()))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_running_maximum_starts_at_zero(device):
+    """Gates far below zero at the first tokens: a maximum that started at
+    minus infinity would follow them down and change the floor."""
+    dev = torch.device(device)
+    H = 2
+    gz = torch.tensor([[-30.0, -30.0, 5.0, 5.0], [-30.0, 2.0, 5.0, 5.0], [1.0, -30.0, -3.0, 5.0]],
+                      device=dev)
+    z = torch.zeros(H, device=dev)
+    mst = torch.full((2, H), 7.0, device=dev)
+    cu, pos = _meta([3], [0], dev)
+    tok, floor = seqmix.exp_gate_scan(gz, z, z, 50.0, mst, torch.tensor([0], dtype=torch.int32,
+                                                                         device=dev), cu, pos)
+    li = 50.0 * torch.tanh(gz[:, :H].double().cpu() / 50.0)
+    lf = torch.nn.functional.logsigmoid(50.0 * torch.tanh(gz[:, H:].double().cpu() / 50.0))
+    m = torch.zeros(H, dtype=F64)
+    for t in range(3):
+        m1 = torch.maximum(lf[t] + m, li[t])
+        assert (tok[t, :, 0].cpu().double() - torch.exp(lf[t] + m - m1)).abs().max() < 1e-5
+        assert (tok[t, :, 1].cpu().double() - torch.exp(li[t] - m1)).abs().max() < 1e-5
+        assert ((floor[t].cpu().double() - torch.exp(-m1)) / torch.exp(-m1)).abs().max() < 1e-5
+        m = m1
+    assert (mst[0].cpu().double() - m).abs().max() < 1e-5
+    assert float(tok[0, 0, 1]) < 1e-9        # 1 if the maximum had followed the gate down
+
+
+def _delta_case(device, m, cuts, dtype=torch.float32, seed=4, lens=(37, 1, 9)):
+    H, G, D, Dv, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+    d = 24
+    g = torch.Generator().manual_seed(seed)
+    cfg = O.make_config([(O.parallel(O.window_attn(), m), None)], width=d)
+    sd = O.make_weights(cfg, seed)
+    hs = [torch.randn(n, d, generator=g).to(dtype).float() for n in lens]
+    p = "l0.mix.right."
+    want = [O.mixer_gated_delta({k: v.double() for k, v in sd.items()}, p, m, h.double(), 1e-5)
+            for h in hs]
+    dev = torch.device(device)
+    C = 2 * G * D + H * Dv
+    w_in = torch.cat([sd[p + n] for n in "qkvg"]).to(dev, dtype)
+    w_g = torch.cat([sd[p + "b"], sd[p + "a"]]).to(dev)
+    conv = torch.cat([sd[p + n + ".conv"] for n in "qkv"]).t().contiguous().to(dev)
+    state = torch.full((len(lens) + 1, H, Dv, D), 9.0, device=dev)
+    tail = torch.full((len(lens) + 1, K - 1, C), -7.0, device=dev)
+    slots = torch.tensor([2, 0, 1][:len(lens)], dtype=torch.int32, device=dev)
+    a_neg = -torch.exp(sd[p + "A_log"]).to(dev)
+    at = [0] * len(lens)
+    got = [[] for _ in lens]
+    k = 0
+    while any(a < n for a, n in zip(at, lens)):
+        feeds = [min(cuts[(k + b) % len(cuts)], n - a) for b, (a, n) in enumerate(zip(at, lens))]
+        cu, pos = _meta(feeds, at, dev)
+        h = torch.cat([hs[b][a:a + f] for b, (a, f) in enumerate(zip(at, feeds))]).to(dev, dtype)
+        u = torch.nn.functional.linear(h, w_in)
+        gz = torch.nn.functional.linear(h.float(), w_g)
+        act, tok = seqmix.delta_prep(u, gz, G, D, H, Dv, conv, tail, a_neg, sd[p + "dt_bias"].to(dev),
+                                     slots, cu, pos)
+        if K > 1:
+            seqmix.seq_state_save(None, u, None, tail, slots, cu, pos)
+        o = seqmix.delta_scan(act, H, D, Dv, 0, G * D, 2 * G * D, H // G, state, slots, cu, pos, tok)
+        y = seqmix.gated_rmsnorm(o, sd[p + "norm"].repeat(H).to(dev), u[:, C:C + H * Dv], 1e-5,
+                                 torch.float32, groups=H, gate_act="silu")
+        y = y.cpu().double() @ sd[p + "o"].double().T
+        o0 = 0
+        for b, f in enumerate(feeds):
+            got[b].append(y[o0:o0 + f])
+            o0 += f
+            at[b] += f
+        k += 1
+    return [torch.cat(x) for x in got], want
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[37], [1], [2, 1, 3, 17, 1, 13]], ids=lambda c: str(len(c)))
+@pytest.mark.parametrize("m", [O.delta(), O.delta(3, 1, 5, 3, 1), O.delta(4, 2, 128, 64, 4),
+                               O.delta(2, 2, 72, 33, 2), O.delta(1, 1, 200, 8, 3)],
+                         ids=lambda m: f"{m['dim']}x{m['vdim']}")
+def test_gated_delta_mixer(device, m, cuts):
+    got, want = _delta_case(device, m, cuts)
+    for a, b in zip(got, want):
+        assert (a - b).abs().max() < 3e-4 * max(1.0, float(b.abs().max()))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_delta_rule_overwrites_a_key(device):
+    """With beta = 1, no decay and unit keys, writing a key twice REPLACES its
+    value (a plain additive memory would return the sum)."""
+    dev = torch.device(device)
+    D, Dv = 8, 4
+    k = torch.zeros(3, D)
+    k[0, 1] = k[1, 5] = k[2, 1] = 1.0
+    v = torch.tensor([[1.0, 2, 3, 4], [5, 6, 7, 8], [-1, -2, -3, -4]])
+    act = torch.cat([k, k, v], dim=1).to(dev)
+    tok = torch.tensor([[[1.0, 1.0]]] * 3, device=dev)
+    state = torch.zeros(2, 1, Dv, D, device=dev)
+    cu, pos = _meta([3], [0], dev)
+    o = seqmix.delta_scan(act, 1, D, Dv, 0, D, 2 * D, 1, state,
+                          torch.tensor([0], dtype=torch.int32, device=dev), cu, pos, tok)
+    assert (o.cpu() - v).abs().max() < 1e-6
+
+
+def _paged(k, v, lens, blk, device, seed=0):
+    nb = sum(-(-n // blk) for n in lens) + 2
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(seed)).tolist()
+    kc = torch.full((nb, blk, k[0].shape[1]), 7.0)
+    vc = torch.full((nb, blk, v[0].shape[1]), 7.0)
+    mb = max(-(-n // blk) for n in lens)
+    bt = torch.zeros(len(lens), mb, dtype=torch.int32)
+    for b, n in enumerate(lens):
+        for j in range(-(-n // blk)):
+            page = perm.pop()
+            bt[b, j] = page
+            m = min(blk, n - j * blk)
+            kc[page, :m] = k[b][j * blk:j * blk + m]
+            vc[page, :m] = v[b][j * blk:j * blk + m]
+    return kc.to(device), vc.to(device), bt.to(device)
+
+
+def _sink_case(device, dtype, H, G, D, Dv, window, lens, feeds, mfma=None, spike=None, seed=2,
+               splits=None, low=False):
+    """Sequences of ``lens`` keys whose last ``feeds`` positions are this step's
+    queries, softmax with a zero sink. ``spike`` = (distance back, strength):
+    the key that far behind each query gets a large score. ``low``: every score
+    far below zero, so the sink takes almost all of the weight."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(lens)
+    ks = [torch.randn(n, G * D, generator=g).to(dtype).float() for n in lens]
+    vs = [torch.randn(n, G * Dv, generator=g).to(dtype).float() for n in lens]
+    qs = [torch.randn(n, H * D, generator=g) for n in lens]
+    if low:
+        for b in range(B):
+            ks[b] = ks[b].abs() + 0.5
+            qs[b] = -(qs[b].abs() + 0.5)
+    if spike is not None:
+        back, strength = spike
+        for b, n in enumerate(lens):
+            for i in range(n):
+                j = i - back
+                if j >= 0:
+                    kk = ks[b][j].view(G, D)
+                    qs[b][i] = (kk.repeat_interleave(H // G, 0) * strength / D).reshape(-1)
+    qs = [q.to(dtype).float() for q in qs]
+    kc, vc, bt = _paged(ks, vs, lens, 16, device, seed)
+    starts = [n - f for n, f in zip(lens, feeds)]
+    cu, pos = _meta(feeds, starts, device)
+    q = torch.cat([qs[b][starts[b]:] for b in range(B)])
+    ctx = torch.tensor(lens, dtype=torch.int32, device=device)
+    scale = 1.0 / math.sqrt(D)
+    sink = torch.zeros(H, device=device)
+    got = seqmix.window_attention(q.to(device, dtype), kc.to(dtype), vc.to(dtype), cu, ctx, bt, pos,
+                                  scale, 0.0, window, 0, None, H, G, D, Dv, max(feeds),
+                                  matrix_cores=mfma, max_ctx=max(lens), key_splits=splits, sink=sink)
+    want = []
+    for b, n in enumerate(lens):
+        o = O.attention(qs[b].double().view(n, H, D), ks[b].double().view(n, G, D),
+                        vs[b].double().view(n, G, Dv), scale, window=window, sink=True)
+        want.append(o[starts[b]:].reshape(-1, H * Dv))
+    return got.cpu().double(), torch.cat(want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,G,D,Dv,window", [(4, 2, 16, 16, 5), (3, 3, 8, 24, 64), (6, 1, 64, 64, 37),
+                                             (8, 1, 24, 8, 0), (2, 2, 6, 130, 1)])
+def test_window_attention_with_sink(device, H, G, D, Dv, window):
+    for low in (False, True):
+        got, want = _sink_case(device, torch.float32, H, G, D, Dv, window, [150, 1, 37, 90],
+                               [150, 1, 1, 23], low=low)
+        assert (got - want).abs().max() < 2e-5
+    if device == "cuda":
+        for splits in (2, 5):
+            got, want = _sink_case(device, torch.float32, H, G, D, Dv, window, [700, 3, 64, 65],
+                                   [1, 1, 1, 2], mfma=False, splits=splits, low=True)
+            assert (got - want).abs().max() < 2e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("back", [0, 1, 4, 5, 6, 63, 64, 65, 127, 128, 129])
+def test_window_edges_with_sink(device, back):
+    """A key ``back`` positions behind every query carries almost all of the
+    softmax weight if it is visible, and the sink's share shows when it is not:
+    windows of 5, 64 and 128 keys, in a prompt portion and in single tokens."""
+    for window in (5, 64, 128):
+        for feeds in ([300], [1]):
+            got, want = _sink_case(device, torch.float32, 2, 1, 16, 16, window, [300], feeds,
+                                   spike=(back, 40.0))
+            assert (got - want).abs().max() < 2e-5, (window, feeds)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,G,D,Dv,dims", [(4, 2, 16, 16, 8), (3, 1, 24, 8, 0), (2, 2, 6, 6, 6),
+                                           (5, 5, 64, 32, 16), (1, 1, 130, 130, 2)])
+def test_whole_projection_norm_and_rotation(device, H, G, D, Dv, dims):
+    """q | k | v rows -> RMS norm over the whole q and k projections with
+    weights, rotate-half rotation (through the load-time row permutation), and
+    the paged append; scores against the oracle's q and k."""
+    from loqa_hub_amd.models.vilulix import _head_rows, _pairs_from_halves
+    g = torch.Generator().manual_seed(5)
+    T, blk, base = 11, 4, 50.0
+    u = torch.randn(T, (H + G) * D + G * Dv + 3, generator=g)
+    qn, kn = torch.randn(H * D, generator=g), torch.randn(G * D, generator=g)
+    pos = torch.tensor([0, 1, 2, 3, 4, 9, 10, 11, 12, 30, 31], dtype=torch.int32)
+    slots = torch.tensor([3, 2, 1, 0, 7, 6, 5, 4, -1, 9, 8], dtype=torch.int32)
+    wq = O.rotate_half(O.norm_plain(u[:, :H * D].double(), qn.double(), 1e-4).view(T, H, D), dims,
+                       base, pos)
+    wk = O.rotate_half(O.norm_plain(u[:, H * D:(H + G) * D].double(), kn.double(), 1e-4)
+                       .view(T, G, D), dims, base, pos)
+    per = _pairs_from_halves(dims, D)
+    iq, ik = _head_rows(H, D, 0, per), _head_rows(G, D, 0, per)
+    up = torch.cat([u[:, :H * D][:, iq], u[:, H * D:(H + G) * D][:, ik], u[:, (H + G) * D:]], 1)
+    cs = seqmix.rope_table_pairs(dims, 40, base, None, device) if dims else None
+    kc = torch.zeros(3, blk, G * D, device=device)
+    vc = torch.zeros(3, blk, G * Dv, device=device)
+    q = seqmix.qk_prep_append(up.to(device), H, G, D, Dv, (H + G) * D, cs, dims, 1e-4, None,
+                              pos.to(device), kc, vc, slots.to(device), torch.float32,
+                              qn[iq].to(device), kn[ik].to(device))
+    assert (q.cpu().double().view(T, H, D) - wq[:, :, per]).abs().max() < 1e-5
+    ok = slots >= 0
+    kk = kc.view(-1, G, D)[slots[ok].long()].cpu().double()
+    assert (kk - wk[ok][:, :, per]).abs().max() < 1e-5
+    vv = vc.view(-1, G * Dv)[slots[ok].long()].cpu()
+    assert torch.equal(vv, u[ok][:, (H + G) * D:(H + G) * D + G * Dv])
+
+
+# --------------------------------------------------------- the whole model
+@pytest.mark.parametrize("device", DEVICES)
+def test_residual_after_every_layer_run(device, full_model):
+    cfg, sd = full_model
+    toks = tokens(29, cfg["vocab"], 10)
+    want = []
+    O.forward(cfg, sd, toks, want)
+    eng = engine(cfg, sd, device)
+    max_q, max_ctx, host = eng._meta([eng.open_sequence()], [toks], decode=False)
+    host["logit_idx"] = np.asarray([0], np.int64)
+    meta = eng._build_meta(eng._to_device(host), max_q, max_ctx, False)
+    got = []
+    eng.model.forward(meta, eng.kv, got)
+    assert len(got) == len(want) == 8
+    for r, (a, b) in enumerate(zip(got, want)):
+        assert (a.cpu().double() - b).abs().max() < 2e-4 * float(b.abs().max()), r
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_whole_prompt(device, dtype, full_model):
+    cfg, sd = full_model
+    toks = tokens(70, cfg["vocab"], 11)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, device, dtype)
+    got = eng.step_logits([eng.open_sequence()], [toks], [list(range(len(toks)))])
+    if dtype == torch.float32:
+        assert rel_err(got, want) < TOL[dtype]
+    else:
+        # a width this small averages little of the 16-bit rounding away: the
+        # typical row is what is pinned
+        assert rel_err(got, want, 0.5) < TOL[dtype] and rel_err(got, want) < 0.2
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[1], [2], [3, 2, 7], [16], [17, 1, 1, 30], [5, 64]],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_portions_and_decode(device, cuts, full_model):
+    """Token-by-token decoding and portions of any size (down to two tokens,
+    shorter than the convolutions, across page borders at 16 and window edges
+    at 6 and 20) give the whole prompt's logits."""
+    cfg, sd = full_model
+    toks = tokens(53, cfg["vocab"], 12)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, device)
+    got = feed(eng, eng.open_sequence(), toks, cuts)
+    assert rel_err(got, want) < TOL[torch.float32]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_unequal_batch_and_reuse(device, full_model):
+    """Four unequal requests, portions beside single tokens in one step; two
+    end early and two new ones take over their pages and state slots. Every
+    request's logits equal the ones it gets alone (oracle)."""
+    cfg, sd = full_model
+    V = cfg["vocab"]
+    reqs = {n: tokens(L, V, 20 + i) for i, (n, L) in
+            enumerate([("a", 41), ("b", 1), ("c", 18), ("d", 33), ("e", 25), ("f", 47)])}
+    want = {n: O.forward(cfg, sd, t) for n, t in reqs.items()}
+    eng = engine(cfg, sd, device, max_tokens=192, max_seqs=4)
+    plan = {"a": [7, 1, 1, 16, 2, 1, 13], "b": [1], "c": [2, 15, 1], "d": [16, 16, 1],
+            "e": [3, 1, 21], "f": [30, 1, 16]}
+    at = {n: 0 for n in reqs}
+    live, waiting, got = {}, ["a", "b", "c", "d", "e", "f"], {n: [] for n in reqs}
+    steps = 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            n = waiting.pop(0)
+            live[n] = eng.open_sequence()
+        names = list(live)
+        feeds, wants = [], []
+        for n in names:
+            k = plan[n].pop(0)
+            feeds.append(reqs[n][at[n]:at[n] + k])
+            wants.append(list(range(k)))
+            at[n] += k
+        out = eng.step_logits([live[n] for n in names], feeds, wants)
+        o = 0
+        for n, f in zip(names, feeds):
+            got[n].append(out[o:o + len(f)])
+            o += len(f)
+            if at[n] == len(reqs[n]):
+                eng.close_sequence(live.pop(n))
+        steps += 1
+    assert steps > 5
+    for n in reqs:
+        assert rel_err(torch.cat(got[n]), want[n]) < TOL[torch.float32], n
+    assert eng.kv.pool.free_blocks() == 192 // 16 and eng.kv.slots.free_slots() == 4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_and_pages_reused_clean(device, full_model):
+    """A pool of exactly one request's size, every state tensor and page
+    overwritten with junk between requests: the next request must not see it."""
+    cfg, sd = full_model
+    eng = engine(cfg, sd, device, max_tokens=48, max_seqs=1)
+    for i, n in enumerate([40, 48, 3, 33]):
+        toks = tokens(n, cfg["vocab"], 30 + i)
+        seq = eng.open_sequence()
+        got = feed(eng, seq, toks, [9, 1, 2])
+        eng.close_sequence(seq)
+        assert rel_err(got, O.forward(cfg, sd, toks)) < TOL[torch.float32], i
+        for t in eng.kv.state.values():
+            t.fill_(1e3)
+        for named in eng.kv.rows.values():
+            for t in named.values():
+                t.fill_(-1e3)
+        for a, b in eng.kv.kv_rows.values():
+            a.fill_(50.0), b.fill_(-50.0)
+        for t in eng.kv.latent.values():
+            t.fill_(30.0)
+    assert eng.kv.pool.free_blocks() == 3 and eng.kv.slots.free_slots() == 1
+
+
+LOOPS = {
+    "none": (FULL, None), "whole": (FULL[:4], (0, 4, 3)), "once": (FULL, (2, 5, 1)),
+    "one_layer": (FULL[:3], (2, 3, 4)), "empty": (FULL[:2], (1, 1, 5)), "tail": (FULL, (3, 5, 2)),
+}
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", list(LOOPS))
+def test_repeated_stretch_variants(device, name):
+    """No repetition, the whole stack repeated, a single pass, one parallel
+    layer repeated four times (pages, a state and a tail per pass), an empty
+    stretch, a stretch at the end of the stack."""
+    layers, loop = LOOPS[name]
+    cfg = O.make_config(layers, loop=loop)
+    sd = O.make_weights(cfg, 7)
+    toks = tokens(37, cfg["vocab"], 13)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, device)
+    got = feed(eng, eng.open_sequence(), toks, [20, 1, 3])
+    assert rel_err(got, want) < TOL[torch.float32]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("window", [16, 17, 32, 33, 1])
+def test_window_edges_in_prompts_and_decoding(device, window):
+    """Windows that end on, just before and just after a page border; the keys
+    just inside and just outside pass the edge in portions and in decoding."""
+    layers = [(O.parallel(O.window_attn(heads=2, kv_heads=1, dim=8, vdim=8, window=window, dims=4,
+                                        scale=2.0)), O.dense_ff(16))]
+    cfg = O.make_config(layers, width=16)
+    sd = O.make_weights(cfg, 8)
+    sd["l0.mix.left.q"] *= 3.0          # peaked scores: one key more or less shows
+    toks = tokens(70, cfg["vocab"], 14)
+    want = O.forward(cfg, sd, toks)
+    for cuts in ([70], [40] + [1] * 30, [15, 2, 16]):
+        eng = engine(cfg, sd, device)
+        got = feed(eng, eng.open_sequence(), toks, cuts)
+        assert rel_err(got, want) < TOL[torch.float32], cuts
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_far_key_in_latent_attention(device):
+    """One layer of latent attention whose queries look for a token hundreds of
+    positions back: copy weights make the score of one far key stand out."""
+    layers = [(O.latent(heads=2, dim=8, rot_dim=2, vdim=8, kv_rank=8, q_rank=8, scale=6.0,
+                        base=1e6), None)]
+    cfg = O.make_config(layers, width=16, vocab=40)
+    sd = O.make_weights(cfg, 9)
+    toks = tokens(300, 40, 15)
+    want = O.forward(cfg, sd, toks)
+    for cuts in ([300], [290] + [1] * 10, [130, 2, 59]):
+        eng = engine(cfg, sd, device, max_tokens=304)
+        got = feed(eng, eng.open_sequence(), toks, cuts)
+        assert rel_err(got, want) < TOL[torch.float32], cuts
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens(device, full_model):
+    cfg, sd = full_model
+    for n in (1, 2, 3):
+        toks = tokens(n, cfg["vocab"], 16 + n)
+        eng = engine(cfg, sd, device)
+        got = feed(eng, eng.open_sequence(), toks, [1])
+        assert rel_err(got, O.forward(cfg, sd, toks)) < TOL[torch.float32]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_other_sizes(device, dtype):
+    """Sizes that are unequal where a usual model makes them equal, single
+    heads, one tap, a window of one, scales of 1 and 0, no soft cap, no
+    repeated stretch, odd widths."""
+    layers = [
+        (O.parallel(O.window_attn(heads=1, kv_heads=1, dim=10, vdim=3, window=1, dims=2),
+                    O.delta(heads=1, kv_heads=1, dim=5, vdim=9, conv=1), 1.0, 0.0), None),
+        (O.latent(heads=1, dim=5, rot_dim=6, vdim=3, kv_rank=7, q_rank=5), O.dense_ff(9)),
+        (O.mlstm(heads=1, dim=3, vdim=5, cap=1.0), O.dense_ff(11)),
+        (O.parallel(O.window_attn(heads=6, kv_heads=3, dim=4, vdim=6, window=100, dims=0),
+                    O.delta(heads=6, kv_heads=1, dim=4, vdim=2, conv=5), 0.0, 2.0), O.dense_ff(8)),
+        (O.latent(heads=4, dim=2, rot_dim=8, vdim=7, kv_rank=3, q_rank=20, scale=0.3), None)]
+    cfg = O.make_config(layers, width=20, vocab=31, softcap=0.0)
+    sd = O.make_weights(cfg, 10)
+    toks = tokens(45, 31, 17)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, device, dtype)
+    got = feed(eng, eng.open_sequence(), toks, [19, 1, 2])
+    if dtype == torch.float32:
+        assert rel_err(got, want) < TOL[dtype]
+    else:
+        # a row whose normaliser product nearly cancels moves far under 16-bit
+        # rounding of q: the typical rows are what is pinned
+        assert rel_err(got, want, 0.5) < TOL[dtype] and rel_err(got, want, 0.9) < 0.2
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decode(device):
+    layers = [(O.mlstm(heads=2, dim=8, vdim=8), None),
+              (O.parallel(O.window_attn(heads=2, kv_heads=1, dim=8, vdim=8, window=24, dims=8)),
+               O.dense_ff(16))]
+    cfg = O.make_config(layers, width=16, vocab=40, loop=(0, 2, 2))
+    sd = O.make_weights(cfg, 11)
+    toks = tokens(150, 40, 18)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, device)
+    got = feed(eng, eng.open_sequence(), toks, [10] + [1] * 140)
+    assert rel_err(got, want) < TOL[torch.float32]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_scheduler(device, full_model):
+    """Schema-less requests through ``submit_batch`` (continuous batching:
+    inline prompts, chunked prompts in mixed steps, decode steps) produce the
+    oracle's greedy continuation."""
+    cfg, sd = full_model
+    V = cfg["vocab"]
+    prompts = [tokens(n, V, 40 + i) for i, n in enumerate([5, 90, 23, 70])]
+    n_new = 6
+
+    def greedy(p):
+        seq = list(p)
+        for _ in range(n_new):
+            seq.append(int(O.forward(cfg, sd, seq)[-1].argmax()))
+        return seq[len(p):]
+    want = [greedy(p) for p in prompts]
+    eng = engine(cfg, sd, device, max_tokens=512, max_seqs=4)
+    eng.chunk_prefill = 32          # prompts longer than inline_prefill go in 32-token chunks
+    eng.inline_prefill = 8
+    reqs = [GenRequest(p, None, max_new_tokens=n_new) for p in prompts]
+    try:
+        eng.submit_batch(reqs[:2]).result(timeout=300)
+        f1 = eng.submit_batch(reqs[2:3])
+        f2 = eng.submit_batch(reqs[3:])
+        f1.result(timeout=300), f2.result(timeout=300)
+    finally:
+        eng.stop()
+    for r, w in zip(reqs, want):
+        assert r.done and r.grammar.emitted == w
+    assert eng.kv.slots.free_slots() == 4
+
+
+def test_generate_entry_point(full_model):
+    cfg, sd = full_model
+    p = tokens(12, cfg["vocab"], 50)
+    eng = engine(cfg, sd, "cpu")
+    r = eng.generate([GenRequest(p, None, max_new_tokens=3)])[0]
+    seq = list(p)
+    for _ in range(3):
+        seq.append(int(O.forward(cfg, sd, seq)[-1].argmax()))
+    assert r.grammar.emitted == seq[len(p):]
+
+
+def test_trace_replay_program(tmp_path, full_model):
+    """The replay command on a checkpoint folder: steps on stdin, logits files
+    and ``done`` lines out; a request that sits out a step goes on later."""
+    from loqa_hub_amd.models.loader import write_safetensors
+    cfg, sd = full_model
+    model = tmp_path / "m"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(cfg))
+    write_safetensors({k: v.to(torch.bfloat16) for k, v in sd.items()},
+                      str(model / "model.safetensors"))
+    a, b = tokens(20, cfg["vocab"], 60), tokens(9, cfg["vocab"], 61)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:11], "want": [0, 10]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:8], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[11:], "want": [8]},
+                                {"id": "b", "tokens": b[8:], "want": [0]}], "end": ["a", "b"]},
+    ]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, "-m", "loqa_hub_amd.cli.trace_run", "--model", str(model),
+                        "--dtype", "float32", "--out", str(out), "--max-tokens", "64",
+                        "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                       capture_output=True, cwd=ROOT, timeout=300)
+    assert p.returncode == 0, p.stderr
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == \
+        ["done 0", "done 1", "done 2"]
+    V = cfg["vocab"]
+    wa, wb = O.forward(cfg, sd, a), O.forward(cfg, sd, b)
+    g0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V))
+    g2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V))
+    assert not (out / "1.f32").exists()
+    assert rel_err(g0, wa[[0, 10]]) < TOL[torch.float32]
+    assert rel_err(g2, torch.stack([wa[19], wb[8]])) < TOL[torch.float32]
+
+
+# ------------------------------------------- matrix-core paths (bf16, GPU only)
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,Dv,window", [(4, 2, 64, 64, 0), (6, 2, 128, 128, 48),
+                                             (8, 1, 64, 128, 70), (2, 2, 128, 64, 200)])
+def test_sink_matrix_cores(H, G, D, Dv, window):
+    """The prompt-portion kernel with a sink against the oracle and against the
+    keys-parallel form, also where the sink outweighs every key."""
+    for low in (False, True):
+        lens, feeds = [700, 1, 333, 90, 450], [700, 1, 70, 17, 1]
+        a, want = _sink_case("cuda", torch.bfloat16, H, G, D, Dv, window, lens, feeds, mfma=True,
+                             low=low)
+        b, _ = _sink_case("cuda", torch.bfloat16, H, G, D, Dv, window, lens, feeds, mfma=False,
+                          low=low)
+        scale = float(want.abs().max())
+        assert (a - want).abs().max() < 0.03 * scale and (b - want).abs().max() < 0.03 * scale
+
+
+@pytest.mark.gpu
+def test_serving_sizes_bf16():
+    """A model with matrix-core head sizes in bfloat16: whole prompt, portions
+    and decoding agree with the oracle within 16-bit rounding."""
+    layers = [(O.mlstm(heads=2, dim=64, vdim=64, cap=15.0), O.dense_ff(96)),
+              (O.latent(heads=2, dim=32, rot_dim=32, vdim=64, kv_rank=48, q_rank=64), O.dense_ff(96)),
+              (O.parallel(O.window_attn(heads=4, kv_heads=2, dim=64, vdim=64, window=24, dims=32),
+                          O.delta(heads=2, kv_heads=1, dim=64, vdim=64, conv=4)), O.dense_ff(96))]
+    cfg = O.make_config(layers, width=128, vocab=90, loop=(0, 3, 2))
+    sd = O.make_weights(cfg, 12)
+    toks = tokens(200, 90, 14)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, "cuda", torch.bfloat16, max_tokens=208)
+    for cuts in ([200], [150, 30] + [1] * 20, [33, 2, 70]):
+        seq = eng.open_sequence()
+        got = feed(eng, seq, toks, cuts)
+        eng.close_sequence(seq)
+        assert rel_err(got, want, 0.5) < TOL[torch.bfloat16] and rel_err(got, want, 0.9) < 0.25, cuts
