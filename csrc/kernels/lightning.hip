@@ -179,16 +179,18 @@ __global__ __launch_bounds__(EC * LS_DP) void state_scan_kernel(
   }
 }
 
-// y = rmsnorm(o) * w * sigmoid(gate), or with `silu_first` rmsnorm(o * silu(gate))
-// * w; a row is normalised in `groups` equal parts, each by its own root mean
-// square. One workgroup per (row, part).
+// y = rmsnorm(o) * w * sigmoid(gate) (mode 0), rmsnorm(o * silu(gate)) * w (mode
+// 1: the gate before the norm) or rmsnorm(o) * w * silu(gate) (mode 2); a row is
+// normalised in `groups` equal parts, each by its own root mean square. One
+// workgroup per (row, part).
 template <typename TG, typename TO>
 __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(
     const float* __restrict__ o, const float* __restrict__ w, const TG* __restrict__ gate, long ldg,
-    float eps, TO* __restrict__ y, int n, int groups, int silu_first) {
+    float eps, TO* __restrict__ y, int n, int groups, int mode) {
   __shared__ float scratch[4];
   const size_t r = blockIdx.x;
   const int per = n / groups, c0 = blockIdx.y * per;
+  const bool silu_first = mode == 1;
   float ss = 0.f;
   for (int c = c0 + threadIdx.x; c < c0 + per; c += blockDim.x) {
     float v = o[r * n + c];
@@ -200,7 +202,8 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(
   for (int c = c0 + threadIdx.x; c < c0 + per; c += blockDim.x) {
     const float g = Act<TG>::ld(gate + r * ldg + c);
     const float v = o[r * n + c];
-    Act<TO>::st(y + r * n + c, silu_first ? v * silu_f(g) * inv * w[c] : v * inv * w[c] * sigmoid_f(g));
+    Act<TO>::st(y + r * n + c, silu_first ? v * silu_f(g) * inv * w[c]
+                                          : v * inv * w[c] * (mode == 2 ? silu_f(g) : sigmoid_f(g)));
   }
 }
 
@@ -253,13 +256,13 @@ extern "C" int loqa_state_scan(const void* act, long ld, int H, int D, int Dv, i
 
 extern "C" int loqa_gated_rmsnorm(const void* o, const void* w, const void* gate, int g_dt, long ldg,
                                   float eps, void* y, int y_dt, int T, int n, int groups,
-                                  int silu_first, hipStream_t st) {
+                                  int mode, hipStream_t st) {
   if (T <= 0) return 0;
   if (groups <= 0 || n % groups) return (int)hipErrorInvalidValue;
 #define GO(TG, TO)                                                                            \
   hipLaunchKernelGGL((gated_rmsnorm_kernel<TG, TO>), dim3(T, groups), dim3(256), 0, st,        \
                      (const float*)o, (const float*)w, (const TG*)gate, ldg, eps, (TO*)y, n,   \
-                     groups, silu_first)
+                     groups, mode)
   if (g_dt == 0 && y_dt == 0) GO(bf16_t, bf16_t);
   else if (g_dt == 0) GO(bf16_t, float);
   else if (y_dt == 0) GO(float, bf16_t);

@@ -144,8 +144,8 @@ class VilulixWeights:
         if wdkv.shape != (R + Dr, d) or wuq.shape != (H * (D + Dr), Rq):
             raise ValueError(f"{p}: latent projection shapes do not match the config")
         if m.rot.half and m.rot.dims:
-            per = _pairs_from_halves(m.rot.dims, Dr).to(dev)
-            wdkv = torch.cat([wdkv[:R], wdkv[R:][per]]).contiguous()
+            per = _pairs_from_halves(m.rot.dims, Dr)
+            wdkv = torch.cat([wdkv[:R], wdkv[R:][per.to(dev)]]).contiguous()
             wuq = wuq[_head_rows(H, D + Dr, D, per).to(dev)].contiguous()
         parts = [W(p + "dq"), wdkv, W(p + "g")]
         if parts[0].shape != (Rq, d) or parts[2].shape != (H * Dv, d):
@@ -179,7 +179,7 @@ class VilulixWeights:
                 or qn.numel() != H * D or kn.numel() != G * D:
             raise ValueError(f"{q}: projection shapes do not match the config")
         if a.rot is not None and a.rot.half and a.rot.dims:
-            per = _pairs_from_halves(a.rot.dims, D).to(dev)
+            per = _pairs_from_halves(a.rot.dims, D)
             iq, ik = _head_rows(H, D, 0, per[:a.rot.dims]).to(dev), \
                 _head_rows(G, D, 0, per[:a.rot.dims]).to(dev)
             wq, wk, qn, kn = wq[iq].contiguous(), wk[ik].contiguous(), qn[iq].contiguous(), \
