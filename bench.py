@@ -420,7 +420,7 @@ def main(argv=None) -> int:
                     help="instead of the hub workload: prefill / decode throughput of the language-"
                          "model families (Pipizen beside Llama stacks of equal size, random weights)")
     ap.add_argument("--lm-sizes", default="1b,7b", help="--lm-bench: layer sizes (1b, 7b, tiny)")
-    ap.add_argument("--lm-families", default="pipizen,sodonex,movinex,llama",
+    ap.add_argument("--lm-families", default="pipizen,sodonex,movinex,vilulix,llama",
                     help="--lm-bench: model families to run")
     ap.add_argument("--lm-prompt", type=int, default=2048, help="--lm-bench: prompt tokens")
     ap.add_argument("--lm-batch", type=int, default=8, help="--lm-bench: decoding sequences")

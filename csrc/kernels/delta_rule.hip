@@ -3,12 +3,12 @@
 //
 //   S <- g_t S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
 //
-// delta_prep_kernel: the input stage, one workgroup per token. The q | k | v
-// columns of the projected row pass a causal convolution per channel (weights
-// tap-major, the last tap is the current token's, no bias; rows before the feed
-// from the sequence's tail slot, zeros before position 0, so a reused slot
-// needs no clearing) and SiLU; q and k heads are staged in LDS, a wave per head
-// makes each a unit vector x / sqrt(sum x^2 + 1e-6) (q also times D^(-1/2)).
+// delta_prep_kernel: the input stage, a wave per (token, run of D channels). The
+// q | k | v columns of the projected row pass a causal convolution per channel
+// (weights tap-major, the last tap is the current token's, no bias; rows before
+// the feed from the sequence's tail slot, zeros before position 0, so a reused
+// slot needs no clearing) and SiLU; a run that is a q or k head is made a unit
+// vector x / sqrt(sum x^2 + 1e-6) by one wave reduction (q also times D^(-1/2)).
 // The gate rows give beta = sigmoid(z) and g = exp(a_neg softplus(z + dt_bias)).
 // Everything it writes is f32.
 //
@@ -60,45 +60,56 @@ __device__ __forceinline__ float dr_sum16(float v) {
 }
 
 template <typename TU>
-__global__ __launch_bounds__(256) void delta_prep_kernel(
+__global__ __launch_bounds__(64) void delta_prep_kernel(
     const TU* __restrict__ u, long ldu, const float* __restrict__ gz, int G, int D, int H, int Dv,
     const float* __restrict__ cw, int taps, const float* __restrict__ tail, int nslots,
     const float* __restrict__ a_neg, const float* __restrict__ dt_bias,
     const int* __restrict__ sslots, const int* __restrict__ cu_q, const int* __restrict__ pos,
     int B, float* __restrict__ act, float* __restrict__ tok) {
-  extern __shared__ float qk[];                 // [2 G D] convolved q | k before the unit norm
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, lane = threadIdx.x;
   if (t >= cu_q[B]) return;
   const int b = dr_seq_of_row(cu_q, B, t);
   const int i = t - cu_q[b], p = pos[t], keep = taps - 1;
   const int QK = 2 * G * D, C = QK + H * Dv;
   const float* ts = tail + (size_t)min(max(sslots[b], 0), nslots - 1) * keep * C;
-  for (int h = threadIdx.x; h < H; h += blockDim.x) {
-    const float* z = gz + (size_t)t * 2 * H;
-    tok[((size_t)t * H + h) * 2] = expf(a_neg[h] * dr_softplus(z[H + h] + dt_bias[h]));
-    tok[((size_t)t * H + h) * 2 + 1] = sigmoid_f(z[h]);
-  }
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float acc = 0.f;
-    for (int j = 0; j < taps; ++j) {
-      const int s = keep - j;                   // how many tokens back this tap reads
-      if (p - s < 0) continue;                  // before the sequence's start
-      const float uv = i - s >= 0 ? Act<TU>::ld(u + (size_t)(t - s) * ldu + c)
-                                  : ts[(size_t)(keep + i - s) * C + c];
-      acc += cw[(size_t)j * C + c] * uv;
+  if (blockIdx.y == 0)
+    for (int h = lane; h < H; h += 64) {
+      const float* z = gz + (size_t)t * 2 * H;
+      tok[((size_t)t * H + h) * 2] = expf(a_neg[h] * dr_softplus(z[H + h] + dt_bias[h]));
+      tok[((size_t)t * H + h) * 2 + 1] = sigmoid_f(z[h]);
     }
-    const float y = silu_f(acc);
-    if (c < QK) qk[c] = y; else act[(size_t)t * C + c] = y;
-  }
-  __syncthreads();
-  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float qscale = 1.f / sqrtf((float)D);
-  for (int hd = wid; hd < 2 * G; hd += nw) {
+  const int units = (C + D - 1) / D;            // runs of D channels: the q heads, the k heads, then v
+  constexpr int NC = 8;                         // channels per lane (D <= 512)
+  for (int un = blockIdx.y; un < units; un += gridDim.y) {
+    const int c0 = un * D, n = min(D, C - c0);
+    float y[NC];
     float ss = 0.f;
-    for (int d = lane; d < D; d += 64) ss += qk[hd * D + d] * qk[hd * D + d];
-    ss = wave_sum(ss);
-    const float inv = (hd < G ? qscale : 1.f) / sqrtf(ss + 1e-6f);
-    for (int d = lane; d < D; d += 64) act[(size_t)t * C + hd * D + d] = qk[hd * D + d] * inv;
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int c = c0 + lane + 64 * k;
+      y[k] = 0.f;
+      if (lane + 64 * k < n) {
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+          const int s = keep - j;               // how many tokens back this tap reads
+          if (p - s < 0) continue;              // before the sequence's start
+          const float uv = i - s >= 0 ? Act<TU>::ld(u + (size_t)(t - s) * ldu + c)
+                                      : ts[(size_t)(keep + i - s) * C + c];
+          acc += cw[(size_t)j * C + c] * uv;
+        }
+        y[k] = silu_f(acc);
+        ss += y[k] * y[k];
+      }
+    }
+    float mul = 1.f;
+    if (c0 < QK) {                              // a q or k head: unit length (q also D^(-1/2))
+      ss = wave_sum(ss);
+      mul = (c0 < G * D ? qscale : 1.f) / sqrtf(ss + 1e-6f);
+    }
+#pragma unroll
+    for (int k = 0; k < NC; ++k)
+      if (lane + 64 * k < n) act[(size_t)t * C + c0 + lane + 64 * k] = y[k] * mul;
   }
 }
 
@@ -230,15 +241,16 @@ extern "C" int loqa_delta_prep(const void* u, int u_dt, long ldu, const void* gz
                                const void* sslots, const void* cu_q, const void* pos, int B, int T,
                                void* act, void* tok, hipStream_t st) {
   if (T <= 0) return 0;
-  if (B <= 0 || taps < 1 || nslots <= 0 || G <= 0 || D <= 0 || H <= 0 || Dv <= 0 ||
-      (size_t)2 * G * D * 4 > 64 * 1024)
+  if (B <= 0 || taps < 1 || nslots <= 0 || G <= 0 || D <= 0 || D > 512 || H <= 0 || Dv <= 0)
     return (int)hipErrorInvalidValue;
+  const int units = (2 * G * D + H * Dv + D - 1) / D;
+  // many rows: a wave walks several runs
+  const dim3 grid(T, T >= 4096 ? (units + 3) / 4 : units);
 #define GO(TU)                                                                                   \
-  hipLaunchKernelGGL(delta_prep_kernel<TU>, dim3(T), dim3(256), (size_t)2 * G * D * 4, st,       \
-                     (const TU*)u, ldu, (const float*)gz, G, D, H, Dv, (const float*)cw, taps,   \
-                     (const float*)tail, nslots, (const float*)a_neg, (const float*)dt_bias,     \
-                     (const int*)sslots, (const int*)cu_q, (const int*)pos, B, (float*)act,      \
-                     (float*)tok)
+  hipLaunchKernelGGL(delta_prep_kernel<TU>, grid, dim3(64), 0, st, (const TU*)u, ldu,            \
+                     (const float*)gz, G, D, H, Dv, (const float*)cw, taps, (const float*)tail,  \
+                     nslots, (const float*)a_neg, (const float*)dt_bias, (const int*)sslots,     \
+                     (const int*)cu_q, (const int*)pos, B, (float*)act, (float*)tok)
   if (u_dt == 0) GO(bf16_t); else GO(float);
 #undef GO
   return (int)hipGetLastError();

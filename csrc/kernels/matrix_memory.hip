@@ -51,7 +51,9 @@ __global__ __launch_bounds__(64) void exp_gate_scan_kernel(
     const int nt = min(64, q1 - t0);
     float m_prev = 0.f, m_mine = 0.f;
     for (int j = 0; j < nt; ++j) {
-      const float lij = __shfl(li, j, 64), lfj = __shfl(lf, j, 64);
+      // j is wave-uniform: scalar lane reads, no trip through the LDS crossbar
+      const float lij = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(li), j));
+      const float lfj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lf), j));
       const float m1 = fmaxf(lfj + m, lij);
       if (lane == j) { m_prev = m; m_mine = m1; }
       m = m1;

@@ -6,8 +6,10 @@ For each size a Pipizen stack (latent attention / lightning mixers, dense and
 mixture-of-experts feed-forwards), a Sodonex stack (chunked sigmoid attention
 with token shift and short convolutions, squared-relu experts) and a Movinex
 stack (a Mamba-2 layer, full and sliding-window softmax attention, GeGLU and
-sigmoid-routed experts) run beside a Llama stack of the same width, depth, head count and feed-forward
-width - the framework's plain decoder. Measured per family:
+sigmoid-routed experts) and a Vilulix stack (parallel layers: a matrix memory,
+latent attention with a query latent, sliding-window attention with a sink
+beside a gated delta rule, dense SwiGLU) run beside a Llama stack of the same
+width, depth, head count and feed-forward width - the framework's plain decoder. Measured per family:
 
 * prefill: one prompt of ``P`` tokens through ``LLMEngine.step_logits``;
 * decode: ``B`` sequences at context ``P`` advancing one token per step
@@ -24,10 +26,11 @@ import time
 import numpy as np
 import torch
 
-from ..models.configs import (ChunkAttnConfig, FeedForwardConfig, HybridLayerConfig,
-                              LatentAttnConfig, LightningConfig, LlamaConfig, LoopConfig,
-                              Mamba2Config, MovinexConfig, PipizenConfig, RotaryConfig,
-                              SodonexConfig, SoftmaxAttnConfig)
+from ..models.configs import (ChunkAttnConfig, DeltaRuleConfig, FeedForwardConfig,
+                              HybridLayerConfig, LatentAttnConfig, LightningConfig, LlamaConfig,
+                              LoopConfig, Mamba2Config, MatrixMemoryConfig, MovinexConfig,
+                              ParallelMixerConfig, PipizenConfig, RotaryConfig, SodonexConfig,
+                              SoftmaxAttnConfig, VilulixConfig)
 
 SIZES = {
     # name: (width, layers, heads, head_dim, rot_dim, kv_rank, ff, experts, expert_ff, top)
@@ -87,6 +90,27 @@ def movinex_stack(name: str, vocab: int = 32000, window: int = 1024) -> MovinexC
     layers += [HybridLayerConfig("attention_2", local, moe) for _ in range(max(0, n - 2))]
     return MovinexConfig(f"movinex-{name}", vocab, d, 1e-6, 1.0, tuple(layers),
                          LoopConfig(1, min(3, len(layers)), 1))
+
+
+def vilulix_stack(name: str, vocab: int = 32000, window: int = 1024) -> VilulixConfig:
+    """Four parallel layers, each with a dense SwiGLU beside its mixer: a matrix
+    memory (the Llama stack's heads and head size for q, k and v), latent
+    attention as in the Pipizen stack with a query latent of 3 x the key/value
+    latent and an output gate, and twice a sliding-window attention (4 query
+    heads per key/value head, rotary on half a head, zero sink) beside a gated
+    delta rule (as many value heads, 4 per query/key head, 4 taps)."""
+    d, n, H, D, Dr, R, ff, _, _, _ = SIZES[name]
+    G = max(1, H // 4)
+    mem = MatrixMemoryConfig(H, D, D, 15.0)
+    lat = LatentAttnConfig(H, D, Dr, D, R, (D + Dr) ** -0.5, RotaryConfig(Dr, 10000.0, half=True),
+                           q_rank=3 * R, gate=True)
+    left = SoftmaxAttnConfig(H, G, D, D, D ** -0.5, rot=RotaryConfig(Dr, 10000.0, half=True),
+                             window=window, qk_norm="whole", zero_sink=True)
+    par = ParallelMixerConfig(left, DeltaRuleConfig(H, G, D, D, 4), 1.0, 1.0)
+    mlp = FeedForwardConfig("dense", ff)
+    layers = [HybridLayerConfig("mlstm", mem, mlp), HybridLayerConfig("latent_attention", lat, mlp)]
+    layers += [HybridLayerConfig("parallel", par, mlp) for _ in range(max(0, n - 2))]
+    return VilulixConfig(f"vilulix-{name}", vocab, d, 1e-6, 30.0, tuple(layers))
 
 
 def llama_stack(name: str, vocab: int = 32000) -> LlamaConfig:
@@ -157,7 +181,7 @@ def run(args) -> int:
     sizes = [s for s in args.lm_sizes.split(",") if s]
     for name in sizes:
         fams = {"pipizen": pipizen_stack, "sodonex": sodonex_stack, "movinex": movinex_stack,
-                "llama": llama_stack}
+                "vilulix": vilulix_stack, "llama": llama_stack}
         for fam in [f for f in args.lm_families.split(",") if f]:
             cfg = fams[fam](name)
             if dev.type == "cpu":      # plumbing run: tiny stacks
