@@ -23,7 +23,9 @@
 //   u = beta (v - g r),   o = g s + u c,   S <- g S + k u
 //
 // which is the definition with the read-out folded in (S_new^T q = g S^T q + u
-// k . q). The state is stored with a column's rows side by side ([slots, H, Dv,
+// k . q). c is the same for every column: it is computed once per token group.
+// The decayed state g S is formed while the sum for r is under way, so that one
+// multiply-add per row follows it. The state is stored with a column's rows side by side ([slots, H, Dv,
 // D]), so a wave reads and writes 4 D contiguous floats. The step's tokens are
 // staged TC at a time in LDS (rows zero-padded to 16 MAXD), the next group's
 // values already in flight in registers. The recurrence runs token by token
@@ -113,6 +115,82 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(
   }
 }
 
+// The same stage for bfloat16 rows whose heads are a power-of-two number (up
+// to 64) of 16-byte runs: a lane owns 8 neighbouring channels (one 16-byte
+// load per tap, 32-byte stores), the D / 8 lanes of a head add up their
+// squares through data-parallel moves, a wave covers 512 channels.
+__device__ __forceinline__ float dr_group_sum(float v, int gs) {
+  if (gs >= 2) v += dr_dpp<0xB1>(v);
+  if (gs >= 4) v += dr_dpp<0x4E>(v);
+  if (gs >= 8) v += dr_dpp<0x141>(v);
+  if (gs >= 16) v += dr_dpp<0x140>(v);
+  if (gs >= 32) v += __shfl_xor(v, 16, 64);
+  if (gs >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+__global__ __launch_bounds__(64) void delta_prep_v8_kernel(
+    const bf16_t* __restrict__ u, long ldu, const float* __restrict__ gz, int G, int D, int H, int Dv,
+    const float* __restrict__ cw, int taps, const float* __restrict__ tail, int nslots,
+    const float* __restrict__ a_neg, const float* __restrict__ dt_bias,
+    const int* __restrict__ sslots, const int* __restrict__ cu_q, const int* __restrict__ pos,
+    int B, float* __restrict__ act, float* __restrict__ tok) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  if (t >= cu_q[B]) return;
+  const int b = dr_seq_of_row(cu_q, B, t);
+  const int i = t - cu_q[b], p = pos[t], keep = taps - 1;
+  const int QK = 2 * G * D, C = QK + H * Dv;
+  const float* ts = tail + (size_t)min(max(sslots[b], 0), nslots - 1) * keep * C;
+  if (blockIdx.y == 0)
+    for (int h = lane; h < H; h += 64) {
+      const float* z = gz + (size_t)t * 2 * H;
+      tok[((size_t)t * H + h) * 2] = expf(a_neg[h] * dr_softplus(z[H + h] + dt_bias[h]));
+      tok[((size_t)t * H + h) * 2 + 1] = sigmoid_f(z[h]);
+    }
+  const float qscale = 1.f / sqrtf((float)D);
+  const int lpg = D / 8;                              // lanes per head
+  for (int c = 8 * (blockIdx.y * 64 + lane); c - 8 * lane < C; c += 8 * 64 * gridDim.y) {
+    const bool ok = c < C;                            // whole waves stay in the loop for the sums
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+    if (ok)
+      for (int j = 0; j < taps; ++j) {
+        const int s = keep - j;                       // how many tokens back this tap reads
+        if (p - s < 0) continue;                      // before the sequence's start
+        float f[8];
+        if (i - s >= 0) {
+          unpack8(*reinterpret_cast<const uint4*>(u + (size_t)(t - s) * ldu + c), f);
+        } else {
+          const float* tr = ts + (size_t)(keep + i - s) * C + c;
+          const float4 a = *reinterpret_cast<const float4*>(tr);
+          const float4 d = *reinterpret_cast<const float4*>(tr + 4);
+          f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = d.x; f[5] = d.y; f[6] = d.z; f[7] = d.w;
+        }
+        const float4 w0 = *reinterpret_cast<const float4*>(cw + (size_t)j * C + c);
+        const float4 w1 = *reinterpret_cast<const float4*>(cw + (size_t)j * C + c + 4);
+        acc[0] += w0.x * f[0]; acc[1] += w0.y * f[1]; acc[2] += w0.z * f[2]; acc[3] += w0.w * f[3];
+        acc[4] += w1.x * f[4]; acc[5] += w1.y * f[5]; acc[6] += w1.z * f[6]; acc[7] += w1.w * f[7];
+      }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      acc[k] = silu_f(acc[k]);
+      ss += acc[k] * acc[k];
+    }
+    ss = dr_group_sum(ss, lpg);                       // q / k heads start on multiples of D
+    float mul = 1.f;
+    if (c < QK) mul = (c < G * D ? qscale : 1.f) / sqrtf(ss + 1e-6f);
+    if (ok) {
+      float* o = act + (size_t)t * C + c;
+      *reinterpret_cast<float4*>(o) =
+          make_float4(acc[0] * mul, acc[1] * mul, acc[2] * mul, acc[3] * mul);
+      *reinterpret_cast<float4*>(o + 4) =
+          make_float4(acc[4] * mul, acc[5] * mul, acc[6] * mul, acc[7] * mul);
+    }
+  }
+}
+
 template <int MAXD, int TC, int EC>   // D <= DR_DP * MAXD
 __global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
     const float* __restrict__ act, long ld, int H, int D, int Dv, int q_off, int k_off, int v_off,
@@ -127,7 +205,7 @@ __global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
   __shared__ __attribute__((aligned(16))) float ks[TC * DPAD];
   __shared__ float vs[TC * EC];
   __shared__ float os[TC * EC];
-  __shared__ float gs[TC], bs[TC];
+  __shared__ float gs[TC], bs[TC], cs[TC];
   const int b = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * EC;
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
   if (q1 <= q0) return;
@@ -190,30 +268,55 @@ __global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
     if (tid < TC) { gs[tid] = rg; bs[tid] = rb; }
     __syncthreads();
     if (t0 + TC < q1) fetch(t0 + TC);      // in flight while this group is computed
+    // k . q of every token of the group once for all columns; the decayed
+    // state is formed while the 16-lane sum of S^T k is under way, so that
+    // one multiply-add per row follows the sum
+    for (int i = tid; i < TC * DR_DP; i += NTH) {
+      const int tt = i / DR_DP, pp = i % DR_DP;
+      float c = 0.f;
+#pragma unroll
+      for (int j = 0; j < MAXD; ++j)
+        c += ks[tt * DPAD + pp * MAXD + j] * qs[tt * DPAD + pp * MAXD + j];
+      c = dr_sum16(c);
+      if (pp == 0) cs[tt] = c;
+    }
+    __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
       float4 kc[MAXD / 4], qc[MAXD / 4];
       const float4* k4 = reinterpret_cast<const float4*>(ks + tt * DPAD + dp * MAXD);
       const float4* q4 = reinterpret_cast<const float4*>(qs + tt * DPAD + dp * MAXD);
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) { kc[i] = k4[i]; qc[i] = q4[i]; }
-      float r0 = 0.f, r1 = 0.f, s0 = 0.f, s1 = 0.f, c0 = 0.f, c1 = 0.f;
+      const float g = gs[tt], bt = bs[tt], vv = vs[tt * EC + e], kq = cs[tt];
+      float r0 = 0.f, r1 = 0.f, s0 = 0.f, s1 = 0.f;
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) {
-        r0 += S[4 * i] * kc[i].x;     s0 += S[4 * i] * qc[i].x;     c0 += kc[i].x * qc[i].x;
-        r1 += S[4 * i + 1] * kc[i].y; s1 += S[4 * i + 1] * qc[i].y; c1 += kc[i].y * qc[i].y;
-        r0 += S[4 * i + 2] * kc[i].z; s0 += S[4 * i + 2] * qc[i].z; c0 += kc[i].z * qc[i].z;
-        r1 += S[4 * i + 3] * kc[i].w; s1 += S[4 * i + 3] * qc[i].w; c1 += kc[i].w * qc[i].w;
+        r0 += S[4 * i] * kc[i].x;     r1 += S[4 * i + 1] * kc[i].y;
+        r0 += S[4 * i + 2] * kc[i].z; r1 += S[4 * i + 3] * kc[i].w;
       }
-      const float r = dr_sum16(r0 + r1), sq = dr_sum16(s0 + s1), kq = dr_sum16(c0 + c1);
-      const float g = gs[tt];
-      const float uu = bs[tt] * (vs[tt * EC + e] - g * r);
+      float r = r0 + r1;
+      r += dr_dpp<0xB1>(r);
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) {
-        S[4 * i] = g * S[4 * i] + kc[i].x * uu;
-        S[4 * i + 1] = g * S[4 * i + 1] + kc[i].y * uu;
-        S[4 * i + 2] = g * S[4 * i + 2] + kc[i].z * uu;
-        S[4 * i + 3] = g * S[4 * i + 3] + kc[i].w * uu;
+        s0 += S[4 * i] * qc[i].x;     s1 += S[4 * i + 1] * qc[i].y;
+        s0 += S[4 * i + 2] * qc[i].z; s1 += S[4 * i + 3] * qc[i].w;
       }
+      r += dr_dpp<0x4E>(r);
+#pragma unroll
+      for (int i = 0; i < MAXD; ++i) S[i] *= g;
+      r += dr_dpp<0x141>(r);
+      float sq = s0 + s1;
+      sq += dr_dpp<0xB1>(sq);
+      r += dr_dpp<0x140>(r);
+      sq += dr_dpp<0x4E>(sq);
+      const float uu = bt * (vv - g * r);
+#pragma unroll
+      for (int i = 0; i < MAXD / 4; ++i) {
+        S[4 * i] += kc[i].x * uu;     S[4 * i + 1] += kc[i].y * uu;
+        S[4 * i + 2] += kc[i].z * uu; S[4 * i + 3] += kc[i].w * uu;
+      }
+      sq += dr_dpp<0x141>(sq);
+      sq += dr_dpp<0x140>(sq);
       if (dp == 0) os[tt * EC + e] = g * sq + uu * kq;
     }
     __syncthreads();
@@ -243,7 +346,18 @@ extern "C" int loqa_delta_prep(const void* u, int u_dt, long ldu, const void* gz
   if (T <= 0) return 0;
   if (B <= 0 || taps < 1 || nslots <= 0 || G <= 0 || D <= 0 || D > 512 || H <= 0 || Dv <= 0)
     return (int)hipErrorInvalidValue;
-  const int units = (2 * G * D + H * Dv + D - 1) / D;
+  const int C = 2 * G * D + H * Dv, lpg = D / 8;
+  if (u_dt == 0 && D % 8 == 0 && lpg <= 64 && (lpg & (lpg - 1)) == 0 && C % 8 == 0 &&
+      ldu % 8 == 0 && ((size_t)u & 15) == 0) {
+    const int per = (C + 511) / 512;
+    hipLaunchKernelGGL(delta_prep_v8_kernel, dim3(T, T >= 2048 ? (per + 1) / 2 : per), dim3(64), 0,
+                       st, (const bf16_t*)u, ldu, (const float*)gz, G, D, H, Dv, (const float*)cw,
+                       taps, (const float*)tail, nslots, (const float*)a_neg,
+                       (const float*)dt_bias, (const int*)sslots, (const int*)cu_q,
+                       (const int*)pos, B, (float*)act, (float*)tok);
+    return (int)hipGetLastError();
+  }
+  const int units = (C + D - 1) / D;
   // many rows: a wave walks several runs
   const dim3 grid(T, T >= 4096 ? (units + 3) / 4 : units);
 #define GO(TU)                                                                                   \

@@ -307,6 +307,43 @@ def test_gated_delta_mixer(device, m, cuts):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("G,D,H,Dv,K", [(2, 128, 4, 64, 4), (1, 16, 3, 8, 2), (3, 64, 3, 40, 3),
+                                        (1, 512, 1, 8, 1), (2, 24, 2, 12, 3)])
+def test_delta_input_stage_bf16(device, G, D, H, Dv, K):
+    """The input stage on 16-bit rows (the vectorised form where a head is a
+    power-of-two number of 16-byte runs), whole and in portions with the tail."""
+    dev = torch.device(device)
+    g = torch.Generator().manual_seed(6)
+    C = 2 * G * D + H * Dv
+    T = 21
+    u = torch.randn(T, C + 8, generator=g).to(torch.bfloat16)
+    gz = torch.randn(T, 2 * H, generator=g)
+    conv = (torch.randn(C, K, generator=g) * 0.6)
+    a_neg, dtb = -torch.rand(H, generator=g), torch.randn(H, generator=g)
+    y = O.silu(O.causal_conv(u[:, :C].double(), conv.double()))
+    qk = y[:, :2 * G * D].view(T, 2 * G, D)
+    qk = qk / torch.sqrt((qk * qk).sum(-1, keepdim=True) + 1e-6)
+    qk[:, :G] *= D ** -0.5
+    want = torch.cat([qk.reshape(T, -1), y[:, 2 * G * D:]], 1)
+    wtok = torch.stack([torch.exp(a_neg.double() * torch.nn.functional.softplus(
+        gz[:, H:].double() + dtb.double())), torch.sigmoid(gz[:, :H].double())], -1)
+    tail = torch.full((2, K - 1, C), 5.0, device=dev)
+    slots = torch.tensor([1], dtype=torch.int32, device=dev)
+    at = 0
+    for n in (T,) if K == 1 else (9, 1, 2, 9):
+        cu, pos = _meta([n], [at], dev)
+        uu = u[at:at + n].to(dev)
+        act, tok = seqmix.delta_prep(uu, gz[at:at + n].to(dev).contiguous(), G, D, H, Dv,
+                                     conv.t().contiguous().to(dev), tail, a_neg.to(dev), dtb.to(dev),
+                                     slots, cu, pos)
+        if K > 1:
+            seqmix.seq_state_save(None, uu, None, tail, slots, cu, pos)
+        assert (act.cpu().double() - want[at:at + n]).abs().max() < 2e-5
+        assert (tok.cpu().double() - wtok[at:at + n]).abs().max() < 1e-5
+        at += n
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_delta_rule_overwrites_a_key(device):
     """With beta = 1, no decay and unit keys, writing a key twice REPLACES its
     value (a plain additive memory would return the sum)."""
