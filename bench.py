@@ -418,7 +418,7 @@ def main(argv=None) -> int:
                     help="--mode hub: serve through the DP front end + worker processes at any N")
     ap.add_argument("--lm-bench", action="store_true",
                     help="instead of the hub workload: prefill / decode throughput of the language-"
-                         "model families (Pipizen beside Llama stacks of equal size, random weights)")
+                         "model families (hybrid stacks beside Llama stacks of equal size, random weights)")
     ap.add_argument("--lm-sizes", default="1b,7b", help="--lm-bench: layer sizes (1b, 7b, tiny)")
     ap.add_argument("--lm-families", default="pipizen,sodonex,movinex,vilulix,llama",
                     help="--lm-bench: model families to run")

@@ -748,6 +748,23 @@ def test_generate_entry_point(full_model):
     assert r.grammar.emitted == seq[len(p):]
 
 
+def test_checkpoint_round_trip(tmp_path, full_model):
+    """save -> config.json + safetensors -> registry -> the same logits."""
+    from loqa_hub_amd.models.loader import save_vilulix
+    from loqa_hub_amd.models.registry import lm_config_of_checkpoint, load_lm_weights
+    cfg_json, sd = full_model
+    cfg = lm_config_from_json(cfg_json, "t")
+    save_vilulix(cfg, {k: v.to(torch.bfloat16) for k, v in sd.items()}, str(tmp_path / "ck"))
+    cfg2 = lm_config_of_checkpoint(str(tmp_path / "ck"), "t")
+    assert cfg2 == cfg and family_of(cfg2).name == "vilulix"
+    w = load_lm_weights(cfg2, str(tmp_path / "ck"), "cpu", dtype=torch.float32, max_positions=64)
+    eng = LLMEngine(cfg2, "cpu", weights=w, max_seqs=1, max_seq_len=64, block_size=16, num_blocks=4,
+                    use_graphs=False, dtype=torch.float32)
+    toks = tokens(30, cfg_json["vocab"], 51)
+    got = eng.step_logits([eng.open_sequence()], [toks], [list(range(30))])
+    assert rel_err(got, O.forward(cfg_json, sd, toks)) < TOL[torch.float32]
+
+
 def test_trace_replay_program(tmp_path, full_model):
     """The replay command on a checkpoint folder: steps on stdin, logits files
     and ``done`` lines out; a request that sits out a step goes on later."""
