@@ -323,10 +323,25 @@ class VilulixModel:
     # a step whose longest feed has at least this many tokens takes the
     # matrix-core prompt path of latent attention (bf16 on the GPU)
     prompt_min_q = 32
+    # a step with at least this many tokens runs the sublayers that do not
+    # depend on each other on two HIP streams: the feed-forward (and the
+    # attention side of a parallel mixer) beside the recurrent scan, whose few
+    # long-running waves leave most of the GPU idle. Smaller steps are bound by
+    # launches, and a second stream only adds events to them.
+    overlap_min_tokens = 128
 
     def __init__(self, w: VilulixWeights):
         self.w, self.cfg = w, w.cfg
         self.runs = self.cfg.runs()
+        self._side = None
+
+    def _side_stream(self, T: int):
+        """The second stream for a step of T tokens (default priority), or None."""
+        if self.w.device.type != "cuda" or T < self.overlap_min_tokens:
+            return None
+        if self._side is None:
+            self._side = torch.cuda.Stream(self.w.device)
+        return self._side
 
     # the cache manager sizes its storage from this: one entry per layer RUN
     def cache_spec(self) -> dict:
@@ -360,20 +375,33 @@ class VilulixModel:
         x0 = self.embed(meta.tokens).contiguous()
         x = x0.clone() if cfg.loop is not None else x0
         n = len(self.runs)
+        side = self._side_stream(x.shape[0])
+        main = torch.cuda.current_stream(x.device) if side is not None else None
         ha = hb = None
         if n:
             L = w.layers[self.runs[0][0]]
             ha, hb = seqmix.residual_rms1p(x, [], None, L["norm1"], L["norm2"], eps, dt)
         for r, (i, _) in enumerate(self.runs):
             lc, L = cfg.layers[i], w.layers[i]
+            ff = None
+            if lc.mlp is not None and side is not None:
+                # both norms are on their way: the feed-forward goes to the
+                # second stream while the mixer runs on this one. Every tensor
+                # either stream reads stays referenced until the streams have
+                # joined below, so neither allocator pool hands it out early.
+                side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    ff = self._dense(hb, L)
             if lc.kind == "mlstm":
                 adds = [(self._mlstm(r, lc.mixer, L, ha, meta, cache), 1.0)]
             elif lc.kind == "latent_attention":
                 adds = [(self._latent(r, lc.mixer, L, ha, meta, cache), 1.0)]
             else:
-                adds = self._parallel(r, lc.mixer, L, ha, meta, cache)
+                adds = self._parallel(r, lc.mixer, L, ha, meta, cache, side)
             if lc.mlp is not None:
-                adds.append((self._dense(hb, L), 1.0))
+                adds.append((ff if ff is not None else self._dense(hb, L), 1.0))
+            if side is not None:
+                main.wait_stream(side)
             # the same launch adds the embedding output when the next run opens
             # a later pass of the repeated stretch, and norms for the next layer
             na = nb = extra = None
@@ -414,10 +442,17 @@ class VilulixModel:
         return latent_mix(L, m, ops.linear(cq, L["wq"]), z, cache.latent[r], meta, eps,
                           self.prompt_min_q, gate)
 
-    def _parallel(self, r, m, L, h, meta, cache) -> list:
+    def _parallel(self, r, m, L, h, meta, cache, side=None) -> list:
         u = ops.linear(h, L["w_in"])                       # left q | k | v, right q | k | v | g
-        return [(self._window(r, m.left, L, u, meta, cache), m.left_scale),
-                (self._delta(r, m.right, L, h, u[:, L["r_off"]:], meta, cache), m.right_scale)]
+        if side is None:
+            left = self._window(r, m.left, L, u, meta, cache)
+        else:
+            # the attention side on the second stream, beside the delta rule
+            side.wait_stream(torch.cuda.current_stream(u.device))
+            with torch.cuda.stream(side):
+                left = self._window(r, m.left, L, u, meta, cache)
+        right = self._delta(r, m.right, L, h, u[:, L["r_off"]:], meta, cache)
+        return [(left, m.left_scale), (right, m.right_scale)]
 
     def _window(self, r, a, L, u, meta, cache) -> torch.Tensor:
         H, G, D, Dv = a.heads, a.kv_heads, a.dim, a.vdim
