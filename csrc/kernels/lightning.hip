@@ -226,7 +226,7 @@ extern "C" int loqa_state_scan(const void* act, long ld, int H, int D, int Dv, i
                                int v_off, int hpg, void* state, int nslots,
                                const void* state_slots, const void* cu_q, const void* positions,
                                const void* decay, const void* tok, const void* skip, void* o, int B,
-                               int T, hipStream_t st) {
+                               int T, int col_block, hipStream_t st) {
   if (T <= 0 || B <= 0) return 0;
   if (D > LS_DP * 16 || D <= 0 || Dv <= 0 || hpg <= 0 || H % hpg || (!decay) == (!tok))
     return (int)hipErrorInvalidValue;
@@ -234,7 +234,9 @@ extern "C" int loqa_state_scan(const void* act, long ld, int H, int D, int Dv, i
   // column block: 32 when (sequences x heads x column blocks) fill the GPU,
   // narrower for a lone prompt
   const long wg32 = (long)B * H * ((Dv + 31) / 32);
-  const int ec = wg32 >= 192 ? 32 : (wg32 * 2 >= 192 ? 16 : 8);
+  int ec = wg32 >= 192 ? 32 : (wg32 * 2 >= 192 ? 16 : 8);
+  // a caller that runs other work beside the scan may ask for denser workgroups
+  if (col_block == 8 || col_block == 16 || col_block == 32) ec = col_block;
 #define GO(MD, TCC, ECC)                                                                          \
   hipLaunchKernelGGL((state_scan_kernel<MD, TCC, ECC>), dim3(B, H, (Dv + ECC - 1) / ECC),         \
                      dim3(ECC * LS_DP),                                                           \

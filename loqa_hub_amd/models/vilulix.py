@@ -393,7 +393,7 @@ class VilulixModel:
                 with torch.cuda.stream(side):
                     ff = self._dense(hb, L)
             if lc.kind == "mlstm":
-                adds = [(self._mlstm(r, lc.mixer, L, ha, meta, cache), 1.0)]
+                adds = [(self._mlstm(r, lc.mixer, L, ha, meta, cache, ff is not None), 1.0)]
             elif lc.kind == "latent_attention":
                 adds = [(self._latent(r, lc.mixer, L, ha, meta, cache), 1.0)]
             else:
@@ -418,7 +418,9 @@ class VilulixModel:
         z = ops.linear(hf, w.head)
         return seqmix.softcap_(z, cfg.logit_softcap) if cfg.logit_softcap > 0 else z
 
-    def _mlstm(self, r, m, L, h, meta, cache) -> torch.Tensor:
+    def _mlstm(self, r, m, L, h, meta, cache, beside: bool = False) -> torch.Tensor:
+        """``beside``: other work runs on the second stream meanwhile, so the scan
+        takes the denser grid and leaves compute units to it."""
         H, D, Dv = m.heads, m.dim, m.vdim
         u = ops.linear(h, L["w_in"])                       # q | k | v | g
         gz = ops.linear(h.float(), L["w_gates"])           # f32: input | forget pre-activations
@@ -426,7 +428,8 @@ class VilulixModel:
                                           meta.state_slots, meta.cu_q, meta.positions)
         act = seqmix.matrix_memory_inputs(u, H, D, Dv)
         o = seqmix.state_scan(act, H, D, Dv + 1, 0, H * D, 2 * H * D, 1, cache.state[r],
-                              meta.state_slots, meta.cu_q, meta.positions, tok=tok)
+                              meta.state_slots, meta.cu_q, meta.positions, tok=tok,
+                              col_block=16 if beside else 0)
         y = seqmix.normalized_gated_rmsnorm(o, floor, L["norm"],
                                             u[:, L["g_off"]:L["g_off"] + H * Dv],
                                             self.cfg.norm_eps, self.w.dtype, H, Dv)

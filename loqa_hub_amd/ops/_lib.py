@@ -218,7 +218,7 @@ _SEQMIX_SIGS = {
     "loqa_latent_prefill": [_vp, _l, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _vp],
     "loqa_lightning_prep": [_vp, _i, _l, _i, _i, _vp, _vp],
     "loqa_state_scan": [_vp, _l, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp,
-                        _vp, _i, _i, _vp],
+                        _vp, _i, _i, _i, _vp],
     "loqa_gated_rmsnorm": [_vp, _vp, _vp, _i, _l, _f, _vp, _i, _i, _i, _i, _i, _vp],
     "loqa_act_mul_any": [_vp, _i, _i, _i, _i, _vp, _vp],
     "loqa_moe_route": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp],

@@ -268,7 +268,8 @@ def lightning_scan(qkv: torch.Tensor, H: int, D: int, Dv: int, state: torch.Tens
 def state_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: int, v_off: int,
                hpg: int, state: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
                positions: torch.Tensor, decay: torch.Tensor | None = None,
-               tok: torch.Tensor | None = None, skip: torch.Tensor | None = None) -> torch.Tensor:
+               tok: torch.Tensor | None = None, skip: torch.Tensor | None = None,
+               col_block: int = 0) -> torch.Tensor:
     """The linear recurrence with a carried matrix state that decayed linear
     attention and Mamba-2 layers share, per sequence and head, token by token
     in f32:  S <- a S + k (c v)^T,  o = S^T q + skip_h v,  with a = ``decay[h]``
@@ -276,7 +277,10 @@ def state_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: in
     [T, W]: head h reads q at ``q_off + (h // hpg) D``, k at ``k_off + (h // hpg)
     D`` and v at ``v_off + h Dv``. ``state`` [slots, H, D, Dv] f32 carries S
     between steps (zero when the step's first position is 0). One kernel and
-    one order of operations for prompt portions and single tokens."""
+    one order of operations for prompt portions and single tokens.
+    ``col_block`` (8, 16 or 32; 0: chosen from the batch) sets the value columns
+    per workgroup: a caller that runs other work beside the scan asks for the
+    denser grid. The result does not depend on it."""
     if not act.is_cuda:
         return ref.state_scan(act, H, D, Dv, q_off, k_off, v_off, hpg, state, state_slots, cu_q,
                               positions, decay, tok, skip)
@@ -303,7 +307,7 @@ def state_scan(act: torch.Tensor, H: int, D: int, Dv: int, q_off: int, k_off: in
         check(kernels().loqa_state_scan(ptr(act), W, H, D, Dv, q_off, k_off, v_off, hpg, ptr(state),
                                         state.shape[0], ptr(state_slots), ptr(cu_q), ptr(positions),
                                         ptr(decay), ptr(tok), ptr(skip), ptr(o), B, T,
-                                        stream_ptr(act)), "state_scan")
+                                        int(col_block), stream_ptr(act)), "state_scan")
     return o
 
 
