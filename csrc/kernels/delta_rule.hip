@@ -14,10 +14,12 @@
 //
 // delta_scan_kernel: one workgroup per (sequence, head, EC value columns). A
 // column of S never meets another column: u_e depends on column e of S only.
-// Sixteen neighbouring lanes share a column, each holding a contiguous run of
-// MAXD of its D rows in registers, so that the two products with the OLD
-// state that a token needs, S^T k and S^T q, are MAXD multiply-adds per lane
-// and one 16-lane sum each through data-parallel moves (no LDS, no barrier):
+// Sixteen neighbouring lanes (thirty-two when there are more than 64 rows)
+// share a column, each holding a contiguous run of MAXD of its D rows in
+// registers, so that the two products with the OLD state that a token needs,
+// S^T k and S^T q, are MAXD multiply-adds per lane and one lane-group sum each
+// through data-parallel moves and, across the two 16-lane rows, the swizzle
+// network (no LDS memory, no barrier):
 //
 //   r = S^T k,  s = S^T q,  c = k . q        (before this token's update)
 //   u = beta (v - g r),   o = g s + u c,   S <- g S + k u
@@ -58,6 +60,15 @@ __device__ __forceinline__ float dr_sum16(float v) {
   v += dr_dpp<0x4E>(v);              // lanes 2 3 0 1 of each four
   v += dr_dpp<0x141>(v);             // the other four of each eight (mirror)
   v += dr_dpp<0x140>(v);             // the other eight of each sixteen (mirror)
+  return v;
+}
+
+// the sum over each run of LPC = 16 or 32 lanes, in every lane of the run; the
+// step across the two 16-lane rows goes through the swizzle network
+template <int LPC> __device__ __forceinline__ float dr_lane_sum(float v) {
+  v = dr_sum16(v);
+  if (LPC == 32)
+    v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));   // lane ^ 16
   return v;
 }
 
@@ -191,14 +202,14 @@ __global__ __launch_bounds__(64) void delta_prep_v8_kernel(
   }
 }
 
-template <int MAXD, int TC, int EC>   // D <= DR_DP * MAXD
-__global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
+template <int MAXD, int TC, int EC, int LPC>   // LPC lanes per column, D <= LPC * MAXD
+__global__ __launch_bounds__(EC * LPC) void delta_scan_kernel(
     const float* __restrict__ act, long ld, int H, int D, int Dv, int q_off, int k_off, int v_off,
     int hpg, float* __restrict__ state, const int* __restrict__ state_slots,
     const int* __restrict__ cu_q, const int* __restrict__ positions, const float* __restrict__ tok,
     float* __restrict__ o) {
-  constexpr int NTH = EC * DR_DP;
-  constexpr int DPAD = DR_DP * MAXD;            // padded row length in LDS
+  constexpr int NTH = EC * LPC;
+  constexpr int DPAD = LPC * MAXD;            // padded row length in LDS
   constexpr int NPT = TC * DPAD / NTH;          // staged q (and k) values per thread
   constexpr int NVT = (TC * EC + NTH - 1) / NTH;
   __shared__ __attribute__((aligned(16))) float qs[TC * DPAD];
@@ -210,7 +221,7 @@ __global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
   if (q1 <= q0) return;
   const int tid = threadIdx.x;
-  const int dp = tid % DR_DP, e = tid / DR_DP;
+  const int dp = tid % LPC, e = tid / LPC;
   const bool col = e0 + e < Dv;
   // a column's rows side by side: state [slots, H, Dv, D]
   float* Sg = state + (((size_t)state_slots[b] * H + h) * Dv + e0 + e) * D + dp * MAXD;
@@ -271,13 +282,13 @@ __global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
     // k . q of every token of the group once for all columns; the decayed
     // state is formed while the 16-lane sum of S^T k is under way, so that
     // one multiply-add per row follows the sum
-    for (int i = tid; i < TC * DR_DP; i += NTH) {
-      const int tt = i / DR_DP, pp = i % DR_DP;
+    for (int i = tid; i < TC * LPC; i += NTH) {
+      const int tt = i / LPC, pp = i % LPC;
       float c = 0.f;
 #pragma unroll
       for (int j = 0; j < MAXD; ++j)
         c += ks[tt * DPAD + pp * MAXD + j] * qs[tt * DPAD + pp * MAXD + j];
-      c = dr_sum16(c);
+      c = dr_lane_sum<LPC>(c);
       if (pp == 0) cs[tt] = c;
     }
     __syncthreads();
@@ -294,29 +305,23 @@ __global__ __launch_bounds__(EC * DR_DP) void delta_scan_kernel(
         r0 += S[4 * i] * kc[i].x;     r1 += S[4 * i + 1] * kc[i].y;
         r0 += S[4 * i + 2] * kc[i].z; r1 += S[4 * i + 3] * kc[i].w;
       }
-      float r = r0 + r1;
-      r += dr_dpp<0xB1>(r);
+      // the decayed state and the second product are formed while the lane sum
+      // of the first is under way
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) {
         s0 += S[4 * i] * qc[i].x;     s1 += S[4 * i + 1] * qc[i].y;
         s0 += S[4 * i + 2] * qc[i].z; s1 += S[4 * i + 3] * qc[i].w;
       }
-      r += dr_dpp<0x4E>(r);
+      const float r = dr_lane_sum<LPC>(r0 + r1);
 #pragma unroll
       for (int i = 0; i < MAXD; ++i) S[i] *= g;
-      r += dr_dpp<0x141>(r);
-      float sq = s0 + s1;
-      sq += dr_dpp<0xB1>(sq);
-      r += dr_dpp<0x140>(r);
-      sq += dr_dpp<0x4E>(sq);
       const float uu = bt * (vv - g * r);
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) {
         S[4 * i] += kc[i].x * uu;     S[4 * i + 1] += kc[i].y * uu;
         S[4 * i + 2] += kc[i].z * uu; S[4 * i + 3] += kc[i].w * uu;
       }
-      sq += dr_dpp<0x141>(sq);
-      sq += dr_dpp<0x140>(sq);
+      const float sq = dr_lane_sum<LPC>(s0 + s1);
       if (dp == 0) os[tt * EC + e] = g * sq + uu * kq;
     }
     __syncthreads();
@@ -387,19 +392,25 @@ extern "C" int loqa_delta_scan(const void* act, long ld, int H, int D, int Dv, i
   // columns: 648 us with 8 columns, 549 us with 16, 586 us with 32) - and the
   // denser grid leaves compute units to whatever runs on the other stream.
   const int ec = Dv > 8 ? 16 : (Dv > 4 ? 8 : 4);
-#define GO(MD, TCC, ECC)                                                                          \
-  hipLaunchKernelGGL((delta_scan_kernel<MD, TCC, ECC>), dim3(B, H, (Dv + ECC - 1) / ECC),         \
-                     dim3(ECC * DR_DP), 0, st, (const float*)act, ld, H, D, Dv, q_off, k_off,     \
+#define GOL(MD, TCC, ECC, LL)                                                                     \
+  hipLaunchKernelGGL((delta_scan_kernel<MD, TCC, ECC, LL>), dim3(B, H, (Dv + ECC - 1) / ECC),     \
+                     dim3(ECC * LL), 0, st, (const float*)act, ld, H, D, Dv, q_off, k_off,        \
                      v_off, hpg, (float*)state, (const int*)state_slots, (const int*)cu_q,        \
                      (const int*)positions, (const float*)tok, (float*)o)
+#define GO(MD, TCC, ECC) GOL(MD, TCC, ECC, 16)
 #define GOE(MD, TCC)                                                                              \
   do {                                                                                            \
     if (ec == 16) GO(MD, TCC, 16); else if (ec == 8) GO(MD, TCC, 8); else GO(MD, TCC, 4);         \
   } while (0)
+  // more than 64 rows: 32 lanes per column (measured on the same prompt: 553 us
+  // with 16 lanes x 8 rows, 501 us with 32 lanes x 4 rows)
   if (D <= 64) GOE(4, 16);
+  else if (ec == 16 && D <= 128) GOL(4, 16, 16, 32);
+  else if (ec == 16) GOL(8, 16, 16, 32);
   else if (D <= 128) GOE(8, 16);
   else GOE(16, 8);
 #undef GOE
 #undef GO
+#undef GOL
   return (int)hipGetLastError();
 }
