@@ -298,7 +298,7 @@ def _delta_case(device, m, cuts, dtype=torch.float32, seed=4, lens=(37, 1, 9)):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("cuts", [[37], [1], [2, 1, 3, 17, 1, 13]], ids=lambda c: str(len(c)))
 @pytest.mark.parametrize("m", [O.delta(), O.delta(3, 1, 5, 3, 1), O.delta(4, 2, 128, 64, 4),
-                               O.delta(2, 2, 72, 33, 2), O.delta(1, 1, 200, 8, 3)],
+                               O.delta(2, 2, 72, 33, 2), O.delta(1, 1, 200, 8, 3), O.delta(2, 1, 160, 24, 2)],
                          ids=lambda m: f"{m['dim']}x{m['vdim']}")
 def test_gated_delta_mixer(device, m, cuts):
     got, want = _delta_case(device, m, cuts)
