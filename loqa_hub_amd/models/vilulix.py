@@ -340,7 +340,8 @@ class VilulixModel:
         if self.w.device.type != "cuda" or T < self.overlap_min_tokens:
             return None
         if self._side is None:
-            self._side = torch.cuda.Stream(self.w.device)
+            from ..utils.streams import placed_stream
+            self._side = placed_stream(self.w.device, "mixer")
         return self._side
 
     # the cache manager sizes its storage from this: one entry per layer RUN

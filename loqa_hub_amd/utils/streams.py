@@ -71,7 +71,12 @@ def aligned_pool_stream(device: torch.device, priority: int, slot: int):
 # The PCM stream-in copies (engine/pcm_staging.py) take the old prefill
 # worker's slot 3: a queue of their own beside the decoders (the copies run on
 # the DMA engine and hold no CU).
-DEFAULT_SLOTS = {"llm": 2, "stt": 30, "encoder": 28, "prefill": 3, "tts": 29, "h2d": 3}
+# "mixer": the second stream of a hybrid decoder's prompt passes (independent
+# sublayers beside the recurrent scans, models/vilulix.py). Measured on a
+# 2048-token prompt issued from the default stream: slots 5 - 7 overlap fully
+# (3.15 - 3.19 ms), slots 0 - 2 a little less (3.23 - 3.26 ms), slots 3 and 4
+# share the issuing stream's hardware queue and do not overlap at all (3.6 ms).
+DEFAULT_SLOTS = {"llm": 2, "stt": 30, "encoder": 28, "prefill": 3, "tts": 29, "h2d": 3, "mixer": 5}
 
 
 def init_pools(device: torch.device) -> None:
